@@ -1,0 +1,197 @@
+"""Benchmark of the deformable-convolution hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c4] [--no-cpu]
+
+A step is one forward + backward (grad input, grad offset, grad weight) of one layer through the
+package's autograd Function on synthetic inputs already resident in HBM.  The default workload is
+BASELINE.json's headline configuration c4: deform3d float32, N=4, 64->64 channels, 16x56x56,
+kernel 3x3x3, stride 1, pad 1, one deformable group, offsets U[-1.5, 1.5].
+
+Prints one JSON line.  `value` is effective TFLOP/s = 3 * 2*N*C_out*(C_in/G)*kV*outV / step time
+(only the three dense contractions are counted as work).  `roofline` describes the slowest kernel
+of the step, timed on its own with HIP events on the stream it is launched on; `cpu_baseline` is
+the CPU oracle (the reference algorithm restated: im2col + GEMM per sample and group) timed on a
+bounded sample of the same workload on the host cores.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}     # MI355X dense matrix peaks
+PEAK_HBM_GBS = 8000.0
+
+# name: (nd, N, C_in, C_out, in, k, stride, pad, dil, cpg, groups, offset scale / dist, dtype)
+CONFIGS = {
+    "c1": (2, 2, 8, 8, 16, 3, 1, 1, 1, 8, 1, 1.5, "float64"),
+    "c2": (2, 8, 256, 256, 56, 3, 1, 1, 1, 256, 1, 2.0, "float32"),
+    "c3": (2, 4, 512, 512, 28, 3, 1, 2, 2, 128, 2, "normal_mix", "float32"),
+    "c4": (3, 4, 64, 64, (16, 56, 56), 3, 1, 1, 1, 64, 1, 1.5, "float32"),
+    "c5": (3, 2, 128, 128, (16, 112, 112), 3, (1, 2, 2), 1, 1, 32, 1, 2.0, "float32"),
+}
+DESCR = {
+    "c1": "deform2d f64 N=2 8->8 16x16 k3 p1 (gradcheck shape)",
+    "c2": "deform2d f32 N=8 256->256 56x56 k3 p1",
+    "c3": "deform2d f32 N=4 512->512 28x28 k3 p2 d2 groups2 dg4",
+    "c4": "deform3d f32 N=4 64->64 16x56x56 k3 s1 p1 dg1 offsets U[-1.5,1.5]",
+    "c5": "deform3d f32 N=2 128->128 16x112x112 k3 s(1,2,2) p1 dg4",
+}
+
+
+def gemm_flops(c):
+    N, C_out = c["x"].shape[0], c["w"].shape[0]
+    return 2.0 * N * C_out * c["w"].shape[1] * math.prod(c["k"]) * math.prod(c["outs"])
+
+
+def algorithmic_bytes(c):
+    """Compulsory traffic: every distinct tensor read once, every result written once."""
+    es = c["x"].element_size()
+    nb = lambda t: t.numel() * es
+    out_b = c["gout"].numel() * es
+    fwd = nb(c["x"]) + nb(c["off"]) + nb(c["w"]) + out_b
+    data = out_b + nb(c["x"]) + nb(c["off"]) + nb(c["w"]) + nb(c["x"]) + nb(c["off"])   # + grad_input, grad_offset
+    wgt = out_b + nb(c["x"]) + nb(c["off"]) + nb(c["w"])                                # + grad_weight
+    return dict(forward=fwd, backward_input_offset=data, backward_weight=wgt)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c4", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    import deform_conv3d_pytorch_op_amd as dcn
+    from deform_conv3d_pytorch_op_amd import _lib
+    from deform_conv3d_pytorch_op_amd.functions import _geom
+    from tests.cases import make_case
+
+    spec = CONFIGS[a.config]
+    dtype = getattr(torch, spec[-1])
+    kw = dict(dtype=dtype, seed=0, bias=False)
+    if spec[-2] == "normal_mix":
+        c = make_case(*spec[:-2], 1.0, off_dist="normal_mix", **kw)
+    else:
+        c = make_case(*spec[:-1], **kw)
+    nd = c["nd"]
+    dev = torch.device("cuda:0")
+    fn = dcn.ConvOffset3dFunction if nd == 3 else dcn.ConvOffset2dFunction
+    x, off, w = (c[k].to(dev).requires_grad_(True) for k in ("x", "off", "w"))
+    gout = c["gout"].to(dev)
+    cfg = (c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+
+    def step():
+        x.grad = off.grad = w.grad = None
+        out = fn.apply(x, off, w, None, *cfg)
+        out.backward(gout)
+
+    def fwd_only():
+        with torch.no_grad():
+            fn.apply(x, off, w, None, *cfg)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        fwd_only()
+    torch.cuda.synchronize()
+    ms_fwd = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    F = gemm_flops(c)
+    value = 3 * F / (ms_step * 1e-3) / 1e12
+
+    # ---- per-kernel durations: each C-ABI call between two HIP events on its own stream ------
+    L = _lib.load()
+    suf = "f32" if dtype == torch.float32 else "f64"
+    geom = _geom(nd, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+    nbytes = L.dcn_workspace_bytes(x.element_size(), x.shape[1], w.shape[0], math.prod(c["k"]), c["groups"])
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    out = torch.empty((x.shape[0], w.shape[0]) + c["outs"], dtype=dtype, device=dev)
+    gin, goff, gw = torch.zeros_like(x), torch.empty_like(off), torch.zeros_like(w)
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    xd, od, wd = x.detach(), off.detach(), w.detach()
+    calls = {
+        "forward": lambda: getattr(L, "dcn%dd_forward_%s" % (nd, suf))(
+            xd.data_ptr(), wd.data_ptr(), od.data_ptr(), None, out.data_ptr(), *geom, ws.data_ptr(), nbytes, sp),
+        "backward_input_offset": lambda: getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))(
+            xd.data_ptr(), wd.data_ptr(), od.data_ptr(), gout.data_ptr(), gin.data_ptr(), goff.data_ptr(), *geom,
+            ws.data_ptr(), nbytes, sp),
+        "backward_weight": lambda: getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))(
+            xd.data_ptr(), od.data_ptr(), gout.data_ptr(), gw.data_ptr(), *geom, None, 0, sp),
+    }
+    kernel_ms = {}
+    for name, call in calls.items():
+        for _ in range(2):
+            assert call() == 0, L.dcn_last_error()
+        evs = []
+        for _ in range(a.steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            assert call() == 0, L.dcn_last_error()
+            e1.record(stream)
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        kernel_ms[name] = sum(e0.elapsed_time(e1) for e0, e1 in evs) / len(evs)
+    dominant = max(kernel_ms, key=kernel_ms.get)
+    ab = algorithmic_bytes(c)
+    peak = PEAK_TFLOPS[spec[-1]]
+    achieved = F / (kernel_ms[dominant] * 1e-3) / 1e12
+    roofline = {"kernel": dominant, "bound": "mfma", "achieved": round(achieved, 3), "peak": peak,
+                "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": None,
+                "ms": round(kernel_ms[dominant], 4),
+                "algorithmic_flops": F, "algorithmic_bytes": ab[dominant],
+                "hbm_frac_at_algorithmic_bytes": round(ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+    kernels = {k: {"ms": round(v, 4), "tflops": round(F / (v * 1e-3) / 1e12, 3),
+                   "mfma_frac": round(F / (v * 1e-3) / 1e12 / peak, 4),
+                   "algorithmic_GBps": round(ab[k] / (v * 1e-3) / 1e9, 1)} for k, v in kernel_ms.items()}
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same workload --------------------
+    cpu = None
+    if not a.no_cpu:
+        from oracle import dcn_oracle as orc
+        ns = 1
+        xs, offs, gs = c["x"][:ns].contiguous(), c["off"][:ns].contiguous(), c["gout"][:ns].contiguous()
+        t0 = time.perf_counter()
+        orc.forward(xs, offs, c["w"], None, *cfg, acc64=False)
+        orc.backward(xs, offs, c["w"], gs, None, *cfg, acc64=False)
+        dt = time.perf_counter() - t0
+        threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+        cpu = {"value": round(3 * F * ns / x.shape[0] / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
+               "kind": "port", "seconds": round(dt, 2),
+               "sample": "%d of %d samples of %s, forward + backward once, float accumulate, OpenMP" %
+                         (ns, x.shape[0], a.config)}
+
+    print(json.dumps({
+        "metric": "deform conv fwd+bwd effective TFLOP/s per layer (3 dense contractions counted)",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_step, 4), "fwd_ms": round(ms_fwd, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32" if dtype == torch.float32 else "f64", "data": "synthetic",
+        "config": {"workload": a.config + ": " + DESCR[a.config]},
+        "mfma_frac_whole_step": round(value / peak, 4),
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+    }))
+
+
+if __name__ == "__main__":
+    main()

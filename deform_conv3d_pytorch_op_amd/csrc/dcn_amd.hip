@@ -1,0 +1,266 @@
+// C ABI of libdcn_amd.so (declared in include/dcn_amd.h): argument validation, workspace
+// layout and kernel launches.  No device memory is allocated here and nothing synchronises; all
+// work is enqueued on the caller's stream.
+#include "../../include/dcn_amd.h"
+#include "dcn_kernels.h"
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+namespace {
+
+using namespace dcn;
+
+thread_local std::string g_err;
+
+int fail(int code, const char* msg) {
+    g_err = msg;
+    return code;
+}
+
+
+// Largest re-laid-out weight any call needs; see relayout_weight_kernel for the two layouts.
+template <typename T> void fwd_weight_pad(int M, int Cg, int& MT, int& mchunks, int& Mp, int& Cgp) {
+    const int TN = Mma<T>::TN, KL = Mma<T>::KL;
+    const int mtiles = (M + TN - 1) / TN;
+    MT = mtiles >= 8 ? 8 : (mtiles > 2 ? 4 : mtiles);          // 1, 2, 4 or 8 tiles per wavefront
+    mchunks = (mtiles + MT - 1) / MT;
+    Mp = mchunks * MT * TN;
+    Cgp = Cg + KL;
+}
+template <typename T> void bwd_weight_pad(int M, int Cg, int& Mp, int& Cgp) {
+    Mp = M + Mma<T>::KL;
+    Cgp = Cg + Mma<T>::TN;
+}
+template <typename T> size_t workspace_need(int C_in, int C_out, int kV, int G) {
+    const int M = C_out / G, Cg = C_in / G;
+    int MT, mchunks, Mp, Cgp, Mp2, Cgp2;
+    fwd_weight_pad<T>(M, Cg, MT, mchunks, Mp, Cgp);
+    bwd_weight_pad<T>(M, Cg, Mp2, Cgp2);
+    const size_t a = (size_t)G * kV * Mp * Cgp, b = (size_t)G * kV * Mp2 * Cgp2;
+    return (a > b ? a : b) * sizeof(T);
+}
+
+struct Geometry {   // the reference's argument list, 2-D mapped onto slots 1,2 with a unit length axis
+    int nd, N, C_in, C_out, in[3], out[3], k[3], pad[3], stride[3], dil[3], cpg, G;
+};
+
+// Mirrors shape_check of the reference as far as it can be stated without tensor handles
+// (deform3d/lib/deform_conv3d_cuda.cpp:24-87): the extents must be consistent with each other and
+// with the output-size formula.  Rank and per-tensor size checks live in the Python front end,
+// which owns the tensors.
+int validate(const Geometry& g, Params& P) {
+    if (g.N <= 0 || g.C_in <= 0 || g.C_out <= 0) return fail(DCN_E_ARGUMENT, "batch / channel extents must be positive");
+    if (g.G <= 0 || g.C_in % g.G || g.C_out % g.G) return fail(DCN_E_ARGUMENT, "input c != kernel c");
+    if (g.cpg <= 0 || g.C_in % g.cpg) return fail(DCN_E_ARGUMENT, "off channel");
+    static const char* const omsg[3] = {"error output ll", "error outhh", "error outww"};
+    for (int a = 3 - g.nd; a < 3; ++a) {
+        if (g.in[a] <= 0 || g.k[a] <= 0 || g.stride[a] <= 0 || g.dil[a] <= 0 || g.pad[a] < 0)
+            return fail(DCN_E_ARGUMENT, "input / kernel / stride / dilation extents must be positive, pad non-negative");
+        if (g.in[a] + 2 * g.pad[a] - g.k[a] < 0) return fail(DCN_E_ARGUMENT, omsg[a]);
+        if ((g.in[a] + 2 * g.pad[a] - g.k[a]) / g.stride[a] + 1 != g.out[a]) return fail(DCN_E_ARGUMENT, omsg[a]);
+    }
+    const long long inV = (long long)g.in[0] * g.in[1] * g.in[2], outV = (long long)g.out[0] * g.out[1] * g.out[2];
+    // per-channel offsets are 32-bit inside the kernels (including a bias of up to 4 channels)
+    if (inV > (1ll << 27) || outV > (1ll << 27)) return fail(DCN_E_ARGUMENT, "a single channel exceeds 2^27 voxels");
+    P.nd = g.nd; P.N = g.N; P.C_in = g.C_in; P.C_out = g.C_out; P.G = g.G; P.cpg = g.cpg; P.DG = g.C_in / g.cpg;
+    P.M = g.C_out / g.G; P.Cg = g.C_in / g.G;
+    for (int a = 0; a < 3; ++a) {
+        P.in[a] = g.in[a]; P.out[a] = g.out[a]; P.k[a] = g.k[a];
+        P.pad[a] = g.pad[a]; P.stride[a] = g.stride[a]; P.dil[a] = g.dil[a];
+    }
+    P.inV = (unsigned)inV; P.outV = (unsigned)outV; P.kV = g.k[0] * g.k[1] * g.k[2];
+    P.tiles = P.mchunks = P.Mp = P.Cgp = P.nsplit = P.nctiles = 0;
+    return DCN_OK;
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_err = std::string(what) + ": " + hipGetErrorString(e);
+        return DCN_E_LAUNCH;
+    }
+    return DCN_OK;
+}
+
+template <typename T>
+int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_t s) {
+    const size_t total = (size_t)P.G * P.kV * P.Mp * P.Cgp;
+    const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+    hipLaunchKernelGGL(relayout_weight_kernel<T>, dim3(blocks), dim3(256), 0, s, P, w, wt, channel_fastest);
+    return check_launch("relayout_weight_kernel");
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int ND>
+int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* bias, T* out, void* ws,
+            size_t ws_bytes, hipStream_t s) {
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    if (!in || !w || !off || !out) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    int MT;
+    fwd_weight_pad<T>(P.M, P.Cg, MT, P.mchunks, P.Mp, P.Cgp);
+    if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
+    T* wt = static_cast<T*>(ws);
+    if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
+    const int TN = Mma<T>::TN;
+    P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
+    const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
+    switch (MT) {
+        case 1: hipLaunchKernelGGL((forward_kernel<T, ND, 1>), grid, dim3(WG), 0, s, P, in, off, wt, bias, out); break;
+        case 2: hipLaunchKernelGGL((forward_kernel<T, ND, 2>), grid, dim3(WG), 0, s, P, in, off, wt, bias, out); break;
+        case 4: hipLaunchKernelGGL((forward_kernel<T, ND, 4>), grid, dim3(WG), 0, s, P, in, off, wt, bias, out); break;
+        default: hipLaunchKernelGGL((forward_kernel<T, ND, 8>), grid, dim3(WG), 0, s, P, in, off, wt, bias, out); break;
+    }
+    return check_launch("forward_kernel");
+}
+
+template <typename T, int ND>
+int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* off, const T* gout, T* gin,
+                          T* goff, void* ws, size_t ws_bytes, hipStream_t s) {
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    bwd_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
+    if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
+    T* wt = static_cast<T*>(ws);
+    if (int rc = relayout<T>(P, w, wt, 1, s)) return rc;
+    const int TN = Mma<T>::TN;
+    P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
+    const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
+    hipLaunchKernelGGL((backward_data_kernel<T, ND>), grid, dim3(WG), 0, s, P, in, off, wt, gout, gin, goff);
+    return check_launch("backward_data_kernel");
+}
+
+template <typename T, int ND, int MT>
+int launch_bwd_weight(const Params& P, const T* in, const T* off, const T* gout, T* gw, hipStream_t s) {
+    const int TN = Mma<T>::TN;
+    const size_t lds = (size_t)WAVES * (MT * TN + TN) * (TN + 1) * sizeof(T);
+    auto kern = backward_weight_kernel<T, ND, MT>;
+    if (lds > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit for backward_weight_kernel");
+        }
+    }
+    const dim3 grid((unsigned)P.nsplit, (unsigned)P.kV, (unsigned)(P.nctiles * P.mchunks));
+    hipLaunchKernelGGL(kern, grid, dim3(WG), lds, s, P, in, off, gout, gw);
+    return check_launch("backward_weight_kernel");
+}
+
+template <typename T, int ND>
+int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout, T* gw, hipStream_t s) {
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    const int TN = Mma<T>::TN;
+    const int mtiles = (P.M + TN - 1) / TN;
+    const int MT = mtiles > 2 ? 4 : mtiles;
+    P.mchunks = (mtiles + MT - 1) / MT;
+    // channel tiles: one per TN channels of every (convolution group x deformable group) segment
+    int nct = 0;
+    for (int gg = 0; gg < P.G; ++gg) {
+        const int cg0 = gg * P.Cg, cg1 = cg0 + P.Cg;
+        for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+            const int cb = cg0 > dg * P.cpg ? cg0 : dg * P.cpg;
+            const int ce = cg1 < (dg + 1) * P.cpg ? cg1 : (dg + 1) * P.cpg;
+            nct += (ce - cb + TN - 1) / TN;
+        }
+    }
+    P.nctiles = nct;
+    if ((long long)nct * P.mchunks > 65535) return fail(DCN_E_ARGUMENT, "too many channel tiles for one launch");
+    // split the position reduction so that the grid holds a few thousand workgroups
+    const long long slabs = (long long)P.N * ((P.outV + TN - 1) / TN);
+    const long long other = (long long)P.kV * nct * P.mchunks;
+    long long split = (4096 + other - 1) / other;
+    const long long max_split = (slabs + WAVES - 1) / WAVES;
+    if (split > max_split) split = max_split;
+    if (split < 1) split = 1;
+    P.nsplit = (int)split;
+    switch (MT) {
+        case 1: return launch_bwd_weight<T, ND, 1>(P, in, off, gout, gw, s);
+        case 2: return launch_bwd_weight<T, ND, 2>(P, in, off, gout, gw, s);
+        default: return launch_bwd_weight<T, ND, 4>(P, in, off, gout, gw, s);
+    }
+}
+
+Geometry geo3(int batch, int input_c, int output_c, int input_l, int input_h, int input_w, int output_l,
+              int output_h, int output_w, int kernel_l, int kernel_h, int kernel_w, int pad_l, int pad_h,
+              int pad_w, int stride_l, int stride_h, int stride_w, int dilation_l, int dilation_h,
+              int dilation_w, int cpg, int group) {
+    return Geometry{3, batch, input_c, output_c, {input_l, input_h, input_w}, {output_l, output_h, output_w},
+                    {kernel_l, kernel_h, kernel_w}, {pad_l, pad_h, pad_w}, {stride_l, stride_h, stride_w},
+                    {dilation_l, dilation_h, dilation_w}, cpg, group};
+}
+Geometry geo2(int batch, int input_c, int output_c, int input_h, int input_w, int output_h, int output_w,
+              int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
+              int dilation_w, int cpg, int group) {
+    return Geometry{2, batch, input_c, output_c, {1, input_h, input_w}, {1, output_h, output_w},
+                    {1, kernel_h, kernel_w}, {0, pad_h, pad_w}, {1, stride_h, stride_w},
+                    {1, dilation_h, dilation_w}, cpg, group};
+}
+
+}  // namespace
+
+#define G3_ARGS batch, input_c, output_c, input_l, input_h, input_w, output_l, output_h, output_w, kernel_l, \
+                kernel_h, kernel_w, pad_l, pad_h, pad_w, stride_l, stride_h, stride_w, dilation_l, dilation_h, \
+                dilation_w, channel_per_deformable_group, group
+#define G2_ARGS batch, input_c, output_c, input_h, input_w, output_h, output_w, kernel_h, kernel_w, pad_h, pad_w, \
+                stride_h, stride_w, dilation_h, dilation_w, channel_per_deformable_group, group
+
+extern "C" {
+
+int dcn_version(void) { return 1; }
+const char* dcn_arch(void) { return "gfx950"; }
+const char* dcn_last_error(void) { return g_err.c_str(); }
+
+size_t dcn_workspace_bytes(int elem_size, int input_c, int output_c, int kernel_volume, int group) {
+    if (group <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0) return 0;
+    return elem_size == 8 ? workspace_need<double>(input_c, output_c, kernel_volume, group)
+                          : workspace_need<float>(input_c, output_c, kernel_volume, group);
+}
+
+#define DEFINE_OPS(SUF, T)                                                                                          \
+    int dcn3d_forward_##SUF(const T* input, const T* weight, const T* offset, const T* bias, T* output,             \
+                            DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {                \
+        return forward<T, 3>(geo3(G3_ARGS), input, weight, offset, bias, output, workspace, workspace_bytes,        \
+                             static_cast<hipStream_t>(stream));                                                     \
+    }                                                                                                               \
+    int dcn3d_backward_input_offset_##SUF(const T* input, const T* weight, const T* offset, const T* grad_output,   \
+                                          T* grad_input, T* grad_offset, DCN3D_GEOMETRY, void* workspace,           \
+                                          size_t workspace_bytes, void* stream) {                                   \
+        return backward_input_offset<T, 3>(geo3(G3_ARGS), input, weight, offset, grad_output, grad_input,           \
+                                           grad_offset, workspace, workspace_bytes,                                 \
+                                           static_cast<hipStream_t>(stream));                                       \
+    }                                                                                                               \
+    int dcn3d_backward_weight_##SUF(const T* input, const T* offset, const T* grad_output, T* grad_weight,          \
+                                    DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {        \
+        (void)workspace; (void)workspace_bytes;                                                                     \
+        return backward_weight<T, 3>(geo3(G3_ARGS), input, offset, grad_output, grad_weight,                        \
+                                     static_cast<hipStream_t>(stream));                                             \
+    }                                                                                                               \
+    int dcn2d_forward_##SUF(const T* input, const T* weight, const T* offset, const T* bias, T* output,             \
+                            DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {                \
+        return forward<T, 2>(geo2(G2_ARGS), input, weight, offset, bias, output, workspace, workspace_bytes,        \
+                             static_cast<hipStream_t>(stream));                                                     \
+    }                                                                                                               \
+    int dcn2d_backward_input_offset_##SUF(const T* input, const T* weight, const T* offset, const T* grad_output,   \
+                                          T* grad_input, T* grad_offset, DCN2D_GEOMETRY, void* workspace,           \
+                                          size_t workspace_bytes, void* stream) {                                   \
+        return backward_input_offset<T, 2>(geo2(G2_ARGS), input, weight, offset, grad_output, grad_input,           \
+                                           grad_offset, workspace, workspace_bytes,                                 \
+                                           static_cast<hipStream_t>(stream));                                       \
+    }                                                                                                               \
+    int dcn2d_backward_weight_##SUF(const T* input, const T* offset, const T* grad_output, T* grad_weight,          \
+                                    DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {        \
+        (void)workspace; (void)workspace_bytes;                                                                     \
+        return backward_weight<T, 2>(geo2(G2_ARGS), input, offset, grad_output, grad_weight,                        \
+                                     static_cast<hipStream_t>(stream));                                             \
+    }
+
+DEFINE_OPS(f32, float)
+DEFINE_OPS(f64, double)
+
+}  // extern "C"

@@ -1,0 +1,166 @@
+// Device-side building blocks shared by the deformable-convolution kernels (gfx950 / CDNA4).
+//
+//  * Mma<T>      -- one MFMA tile per data type: v_mfma_f32_32x32x2_f32 for float,
+//                   v_mfma_f64_16x16x4_f64 for double, with the register->row map of the result.
+//  * TapGeo      -- the sampling geometry of one (kernel tap, output position): inside test,
+//                   corner offsets and fractions, following the reference sampler
+//                   (deform3d/lib/deform_conv3d_cuda_kernel.cu:21-26,40-45,123-124 and
+//                   deform2d_double/lib/deform_conv2d_cuda_kernel.cu:31-34,43-46,114-115).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace dcn {
+
+struct Params {
+    int nd;                       // 2 or 3 (informative; kernels are templated on it)
+    int N, C_in, C_out, G, cpg, DG;
+    int M, Cg;                    // output / input channels per convolution group
+    int in[3], out[3], k[3], pad[3], stride[3], dil[3];   // (l,h,w); 2-D uses slots 1,2
+    unsigned inV, outV;           // voxels per channel, input / output
+    int kV;
+    int tiles;                    // position tiles per sample (kernel specific)
+    int mchunks;                  // output-channel chunks handled by separate workgroups
+    int Mp, Cgp;                  // padded extents of the re-laid-out weight in the workspace
+    int nsplit;                   // backward-weight: number of position splits
+    int nctiles;                  // backward-weight: channel tiles over all (group, deformable group) segments
+};
+
+// ---------------------------------------------------------------------------------------------
+template <typename T> struct Mma;
+
+// v_mfma_f32_32x32x2_f32: A is 32x2, B is 2x32, D is 32x32.  Lane l supplies A[l%32][l/32] and
+// B[l/32][l%32]; it receives D[row(r, l/32)][l%32] in 16 registers r, rows grouped in fours.
+template <> struct Mma<float> {
+    static constexpr int TN = 32;     // tile edge (rows of A, columns of B)
+    static constexpr int KL = 2;      // reduction slots spread over lane groups
+    static constexpr int NACC = 16;
+    typedef float Acc __attribute__((ext_vector_type(16)));
+    __device__ static inline Acc mma(float a, float b, Acc c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    __device__ static inline int row(int r, int lg) { return (r >> 2) * 8 + lg * 4 + (r & 3); }
+};
+
+// v_mfma_f64_16x16x4_f64: A is 16x4, B is 4x16, D is 16x16.  Lane l supplies A[l%16][l/16] and
+// B[l/16][l%16]; it receives D[4*r + l/16][l%16] in 4 registers r.
+template <> struct Mma<double> {
+    static constexpr int TN = 16;
+    static constexpr int KL = 4;
+    static constexpr int NACC = 4;
+    typedef double Acc __attribute__((ext_vector_type(4)));
+    __device__ static inline Acc mma(double a, double b, Acc c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    __device__ static inline int row(int r, int lg) { return r * 4 + lg; }
+};
+
+template <typename T> __device__ inline typename Mma<T>::Acc acc_zero() {
+    typename Mma<T>::Acc z;
+#pragma unroll
+    for (int i = 0; i < Mma<T>::NACC; ++i) z[i] = 0;
+    return z;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Axis a of an ND kernel lives in slot a + (3 - ND) of the Params arrays.
+template <int ND> __device__ inline constexpr int slot(int a) { return a + 3 - ND; }
+
+template <int ND>
+__device__ inline void decode_pos(const Params& P, unsigned pos, int o[ND]) {
+    if (ND == 3) {
+        o[2] = pos % P.out[2];
+        unsigned t = pos / P.out[2];
+        o[1] = t % P.out[1];
+        o[0] = t / P.out[1];
+    } else {
+        o[1] = pos % P.out[2];
+        o[0] = pos / P.out[2];
+    }
+}
+
+template <int ND>
+__device__ inline void decode_tap(const Params& P, int tap, int kk[ND]) {
+    if (ND == 3) {
+        kk[2] = tap % P.k[2];
+        int t = tap / P.k[2];
+        kk[1] = t % P.k[1];
+        kk[0] = t / P.k[1];
+    } else {
+        kk[1] = tap % P.k[2];
+        kk[0] = tap / P.k[2];
+    }
+}
+
+template <typename T, int ND>
+struct TapGeo {
+    static constexpr int NC = 1 << ND;
+    unsigned idx[NC];   // voxel offset of each corner inside one channel; corner bit (ND-1-a) = high on axis a
+    T f[ND];            // fraction toward the high corner on each axis
+    T p[ND];            // absolute sampling coordinate
+    bool inside;        // strict -1 < p < size on every axis
+};
+
+// `off_tap` points at offset[n][dg][tap][0][0]; `ib[a]` is out*stride - pad of this lane's
+// position, `kd[a]` is tap*dilation (wave-uniform).  Corner indices are only meaningful when
+// `inside`; otherwise they are zero so that a masked-off lane never forms a wild address.
+template <typename T, int ND>
+__device__ inline void tap_setup(const Params& P, const T* __restrict__ off_tap, unsigned pos,
+                                 const int ib[ND], const int kd[ND], TapGeo<T, ND>& t) {
+    bool inside = true;
+    int lo[ND], hi[ND];
+#pragma unroll
+    for (int a = 0; a < ND; ++a) {
+        const int size = P.in[slot<ND>(a)];
+        // integer part formed in int and converted once, then the offset is added (reference:
+        // `l_in + l_kernel*dilation_l + data_offset_base_ptr[...]`)
+        const T p = (T)(ib[a] + kd[a]) + off_tap[(size_t)a * P.outV + pos];
+        t.p[a] = p;
+        inside = inside && (p > (T)-1) && (p < (T)size);
+        const int l = (int)p;                                   // truncation toward zero
+        lo[a] = l;
+        hi[a] = (p >= (T)(size - 1) || p <= (T)0) ? l : l + 1;  // rim: high corner collapses
+        t.f[a] = p - (T)l;
+    }
+    t.inside = inside;
+    if (ND == 3) {
+        const unsigned s1 = P.in[2], s2 = P.in[1] * P.in[2];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int l = (c & 4) ? hi[0] : lo[0], h = (c & 2) ? hi[1] : lo[1], w = (c & 1) ? hi[2] : lo[2];
+            t.idx[c] = inside ? (unsigned)l * s2 + (unsigned)h * s1 + (unsigned)w : 0u;
+        }
+    } else {
+        const unsigned s1 = P.in[2];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int h = (c & 2) ? hi[0] : lo[0], w = (c & 1) ? hi[1] : lo[1];
+            t.idx[c] = inside ? (unsigned)h * s1 + (unsigned)w : 0u;
+        }
+    }
+}
+
+// Interpolated value of one channel: lerp along w, then h, then l (reference order,
+// deform3d kernel.cu:48-56, deform2d_double kernel.cu:50-53).  `chan` points at the channel's
+// first voxel; `voff` are the corner offsets (possibly biased by the caller, see kernels).
+template <typename T, int ND>
+__device__ inline T sample(const T* __restrict__ chan, const unsigned* voff, const T* f) {
+    if (ND == 3) {
+        const T c000 = chan[voff[0]], c001 = chan[voff[1]], c010 = chan[voff[2]], c011 = chan[voff[3]];
+        const T c100 = chan[voff[4]], c101 = chan[voff[5]], c110 = chan[voff[6]], c111 = chan[voff[7]];
+        const T fw = f[2], gw = (T)1 - fw, fh = f[1], gh = (T)1 - fh, fl = f[0], gl = (T)1 - fl;
+        const T c00 = c000 * gw + c001 * fw, c01 = c010 * gw + c011 * fw;
+        const T c10 = c100 * gw + c101 * fw, c11 = c110 * gw + c111 * fw;
+        const T c0 = c00 * gh + c01 * fh, c1 = c10 * gh + c11 * fh;
+        return c0 * gl + c1 * fl;
+    } else {
+        const T c00 = chan[voff[0]], c01 = chan[voff[1]], c10 = chan[voff[2]], c11 = chan[voff[3]];
+        const T fw = f[1], gw = (T)1 - fw, fh = f[0], gh = (T)1 - fh;
+        const T c0 = c00 * gw + c01 * fw, c1 = c10 * gw + c11 * fw;
+        return c0 * gh + c1 * fh;
+    }
+}
+
+__device__ inline void atomic_add(float* p, float v) { unsafeAtomicAdd(p, v); }
+__device__ inline void atomic_add(double* p, double v) { unsafeAtomicAdd(p, v); }
+
+}  // namespace dcn

@@ -1,0 +1,362 @@
+// Deformable-convolution kernels for gfx950.  All three are implicit GEMMs: the sampled column
+// buffer [C_in*kV, outV] of the reference (deform3d/lib/deform_conv3d_cuda.cpp:110-148) is
+// produced in registers / LDS and consumed by MFMA in the same kernel; it never reaches HBM.
+//
+// Lane roles.  One wavefront owns TN output positions (TN = 32 for float, 16 for double); lane
+// l works on position l % TN and on reduction slot l / TN.  Offsets, corner indices and
+// fractions of a (tap, position) are computed once per deformable group and reused for all of
+// its channels (the reference recomputes them per channel).
+#pragma once
+#include "dcn_device.h"
+
+namespace dcn {
+
+constexpr int WG = 256;            // 4 wavefronts
+constexpr int WAVES = WG / 64;
+
+// ---------------------------------------------------------------------------------------------
+// Weight re-layout into the workspace (tiny: the whole weight is at most a few MB).
+//  forward:        Wt[g][tap][cl][m]   (m fastest, padded to Mp; cl padded to Cgp)  -> MFMA A rows = m
+//  backward-data:  Wt[g][tap][m][cl]   (cl fastest, padded to Cgp; m padded to Mp)  -> MFMA A rows = channels
+// Padding is zero so that reduction slots past the end contribute nothing.
+template <typename T>
+__global__ void relayout_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wt, int channel_fastest) {
+    const size_t total = (size_t)P.G * P.kV * P.Mp * P.Cgp;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        int m, cl;
+        size_t t;
+        if (channel_fastest) { cl = i % P.Cgp; t = i / P.Cgp; m = t % P.Mp; t /= P.Mp; }
+        else                 { m = i % P.Mp;  t = i / P.Mp;  cl = t % P.Cgp; t /= P.Cgp; }
+        const int tap = t % P.kV, g = t / P.kV;
+        T v = 0;
+        if (m < P.M && cl < P.Cg) v = W[(((size_t)g * P.M + m) * P.Cg + cl) * P.kV + tap];
+        Wt[i] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Forward: out[n][g*M + m][pos] = sum_{cl,tap} W[g*M+m][cl][tap] * sample(in[n][g*Cg+cl], tap, pos)  (+ bias)
+// replaces deformable_im2col + the per-group Sgemm (deform3d/lib/deform_conv3d_cuda.cpp:110-148,
+// deform2d_double/lib/deform_conv2d_cuda.cpp:102-138).
+//
+// grid.x = N * tiles (a tile is WAVES*TN consecutive positions of one sample)
+// grid.y = G * mchunks (a chunk is MT*TN output channels)
+// The sampled value of lane (j, q) is the B operand B[k = q][col = j] of the MFMA directly; the
+// A operand comes from the re-laid-out weight.
+template <typename T, int ND, int MT>
+__global__ __launch_bounds__(WG) void forward_kernel(Params P, const T* __restrict__ in,
+                                                     const T* __restrict__ off, const T* __restrict__ Wt,
+                                                     const T* __restrict__ bias, T* __restrict__ out) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % TN, q = lane / TN;
+    const int n = blockIdx.x / P.tiles, tile = blockIdx.x % P.tiles;
+    const int g = blockIdx.y / P.mchunks, mchunk = blockIdx.y % P.mchunks;
+
+    const unsigned pos = (unsigned)(tile * WAVES + wave) * TN + j;
+    const bool valid = pos < P.outV;
+    const unsigned posc = valid ? pos : P.outV - 1;
+    int o[ND], ib[ND];
+    decode_pos<ND>(P, posc, o);
+#pragma unroll
+    for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
+
+    typename MM::Acc acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
+
+    const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
+    for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+        const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
+        const int nsteps = (ce - cb + KL - 1) / KL;
+        const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+        for (int tap = 0; tap < P.kV; ++tap) {
+            int kk[ND], kd[ND];
+            decode_tap<ND>(P, tap, kk);
+#pragma unroll
+            for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+            TapGeo<T, ND> t;
+            tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, posc, ib, kd, t);
+            const bool live = valid && t.inside;
+            if (!__any(live)) continue;        // whole wave outside: the column rows are zero
+            unsigned voff[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
+            const T* chan = in + ((size_t)n * P.C_in + cb) * P.inV;                        // wave-uniform
+            const T* wrow = Wt + (((size_t)g * P.kV + tap) * P.Cgp + (cb - cg0) + q) * P.Mp +
+                            (size_t)mchunk * MT * TN + j;
+            for (int s = 0; s < nsteps; ++s) {
+                T b = 0;
+                if (live && cb + s * KL + q < ce) b = sample<T, ND>(chan, voff, t.f);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wrow[mt * TN], b, acc[mt]);
+                chan += (size_t)KL * P.inV;
+                wrow += (size_t)KL * P.Mp;
+            }
+        }
+    }
+
+    if (!valid) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < MM::NACC; ++r) {
+            const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
+            if (m < P.M) {
+                T v = acc[mt][r];
+                if (bias) v += bias[g * P.M + m];
+                out[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward to input and offset.  Per (tap, TN channels, TN positions) the grad-column tile
+//     gcol[c][pos] = sum_m W[g*M+m][c][tap] * gout[n][g*M+m][pos]
+// is formed by MFMA (replaces the Sgemm at deform3d/lib/deform_conv3d_cuda.cpp:213-220) and lands
+// with lane = position, registers = channels, which is exactly what the two consumers need:
+//   col2im_input  (deform3d kernel.cu:229-296, 2-D deform2d_double kernel.cu:201-238): the value
+//                 is scattered to the 8 (4) corners with weights (w_l*w_h*w_w)*gcol;
+//   col2im_offset (deform3d kernel.cu:386-483, 2-D :309-366): gcol times the derivative of the
+//                 interpolation along each axis, summed over the channels of the deformable group,
+//                 plus -- 3-D only -- the out-of-range branches (:470-481), which compare the h
+//                 and w coordinates against the LENGTH extent exactly like the reference.
+// grid.x = N * tiles, grid.y = DG.  grad_offset gets a plain store of every element.
+template <typename T, int ND>
+__global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __restrict__ in,
+                                                           const T* __restrict__ off, const T* __restrict__ Wt,
+                                                           const T* __restrict__ gout, T* __restrict__ gin,
+                                                           T* __restrict__ goff) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % TN, q = lane / TN;
+    const int n = blockIdx.x / P.tiles, tile = blockIdx.x % P.tiles;
+    const int dg = blockIdx.y;
+
+    const unsigned pos = (unsigned)(tile * WAVES + wave) * TN + j;
+    const bool valid = pos < P.outV;
+    const unsigned posc = valid ? pos : P.outV - 1;
+    int o[ND], ib[ND];
+    decode_pos<ND>(P, posc, o);
+#pragma unroll
+    for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
+
+    const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
+    const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+    T* goff_dg = goff + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+
+    for (int tap = 0; tap < P.kV; ++tap) {
+        int kk[ND], kd[ND];
+        decode_tap<ND>(P, tap, kk);
+#pragma unroll
+        for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+        TapGeo<T, ND> t;
+        tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, posc, ib, kd, t);
+        const bool live = valid && t.inside;
+
+        // corner weights, multiplied in the reference's order (w_l * w_h * w_w)
+        T cw[NC];
+        if (ND == 3) {
+            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+            cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+            cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+        } else {
+            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+            cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+        }
+        // 3-D out-of-range branches: sign per axis for |gcol| (0 = no contribution)
+        T oob[ND];
+#pragma unroll
+        for (int a = 0; a < ND; ++a) oob[a] = 0;
+        if (ND == 3 && valid && !t.inside) {
+            const T len = (T)P.in[0];
+#pragma unroll
+            for (int a = 0; a < 3; ++a) oob[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= len) ? (T)1 : (T)0);
+        }
+        const bool any_oob = (ND == 3) && (oob[0] != 0 || oob[ND - 2] != 0 || oob[ND - 1] != 0);
+        T ga[ND];
+#pragma unroll
+        for (int a = 0; a < ND; ++a) ga[a] = 0;
+
+        if (__any(live || any_oob)) {
+            for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
+                const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
+                const T* gb = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV + posc;
+                for (int c0 = rb; c0 < re; c0 += TN) {
+                    typename MM::Acc d = acc_zero<T>();
+                    const T* wa = Wt + (((size_t)g * P.kV + tap) * P.Mp + q) * P.Cgp + (c0 - g * P.Cg) + j;
+                    const T* gq = gb + (size_t)q * P.outV;
+                    for (int m0 = 0; m0 < P.M; m0 += KL) {
+                        const T a = *wa;
+                        const T b = (valid && m0 + q < P.M) ? *gq : (T)0;
+                        d = MM::mma(a, b, d);
+                        wa += (size_t)KL * P.Cgp;
+                        gq += (size_t)KL * P.outV;
+                    }
+#pragma unroll
+                    for (int r = 0; r < MM::NACC; ++r) {
+                        const int c = c0 + MM::row(r, q);
+                        if (c >= re) continue;
+                        const T gv = d[r];
+                        if (live) {
+                            const T* ic = in + ((size_t)n * P.C_in + c) * P.inV;
+                            T* gc = gin + ((size_t)n * P.C_in + c) * P.inV;
+                            T v[NC];
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
+                            if (ND == 3) {
+                                const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh,
+                                        fw = t.f[2], gw = (T)1 - fw;
+                                const T dl = ((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
+                                             ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh;
+                                const T dh = ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
+                                             ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl;
+                                const T dw = ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                             ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
+                                ga[0] += gv * dl; ga[1] += gv * dh; ga[2] += gv * dw;
+                            } else {
+                                const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                                ga[0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
+                                ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
+                            }
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
+                        } else if (ND == 3 && any_oob) {
+                            const T av = gv > 0 ? gv : -gv;
+#pragma unroll
+                            for (int a = 0; a < ND; ++a) ga[a] += oob[a] * av;
+                        }
+                    }
+                }
+            }
+        }
+        // sum the partial results of the KL lane groups that share a position, then one
+        // coalesced store per axis
+#pragma unroll
+        for (int a = 0; a < ND; ++a) {
+#pragma unroll
+            for (int sh = TN; sh < 64; sh <<= 1) ga[a] += __shfl_xor(ga[a], sh);
+            if (q == 0 && valid) goff_dg[((size_t)tap * ND + a) * P.outV + pos] = ga[a];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward to weight: gW[g*M+m][cl][tap] += sum_{n,pos} gout[n][g*M+m][pos] * sample(in[n][g*Cg+cl], tap, pos)
+// replaces the second deformable_im2col + Sgemm(beta=1) of deform3d/lib/deform_conv3d_cuda.cpp:283-320.
+// The reduction runs over positions, so both MFMA operands need lanes along the non-reduced
+// dimension (m, channel) while memory and the sampler are contiguous along positions: each
+// wavefront transposes its TN-position slab of grad_output and of sampled values through a
+// private LDS region.  A workgroup keeps one (tap, channel tile, m chunk) for its whole life and
+// strides over position slabs, so the [MT*TN x TN] accumulator stays in registers; partial sums
+// of different workgroups meet in grad_weight through hardware float atomics.
+// grid.x = nsplit, grid.y = kV, grid.z = nctiles * mchunks.
+template <typename T, int ND, int MT>
+__global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* __restrict__ in,
+                                                             const T* __restrict__ off,
+                                                             const T* __restrict__ gout, T* __restrict__ gw) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
+    constexpr int LD = TN + 1;                     // padded row: conflict-free transposed reads
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % TN, q = lane / TN;
+    T* sA = reinterpret_cast<T*>(smem_raw) + (size_t)wave * (MT * TN + TN) * LD;   // [MT*TN][LD] grad_output slab
+    T* sB = sA + (size_t)MT * TN * LD;                                            // [TN][LD]    sampled slab
+
+    const int tap = blockIdx.y;
+    const int mchunk = blockIdx.z % P.mchunks;
+    int z = blockIdx.z / P.mchunks;
+    // locate channel tile z: segments are the intersections of convolution groups with deformable groups
+    int g = 0, dg = 0, c0 = 0, ce = 0;
+    bool found = false;
+    for (g = 0; g < P.G && !found; ++g) {
+        const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
+        for (dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+            const int cb = max(cg0, dg * P.cpg);
+            ce = min(cg1, (dg + 1) * P.cpg);
+            const int nt = (ce - cb + TN - 1) / TN;
+            if (z < nt) { c0 = cb + z * TN; found = true; break; }
+            z -= nt;
+        }
+        if (found) break;
+    }
+    if (!found) return;     // uniform for the workgroup
+
+    int kk[ND], kd[ND];
+    decode_tap<ND>(P, tap, kk);
+#pragma unroll
+    for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+
+    typename MM::Acc acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
+
+    const int slabs_per_sample = (P.outV + TN - 1) / TN;
+    const int nslabs = P.N * slabs_per_sample;
+    const int stride_slabs = gridDim.x * WAVES;
+    const int m_base = mchunk * MT * TN;
+    // uniform trip count for all wavefronts of the grid (the barriers below need it)
+    const int trips = (nslabs + stride_slabs - 1) / stride_slabs;
+    for (int it = 0; it < trips; ++it) {
+        const int slab = it * stride_slabs + blockIdx.x * WAVES + wave;
+        const bool slab_ok = slab < nslabs;
+        const int n = slab_ok ? slab / slabs_per_sample : 0;
+        const unsigned p0 = slab_ok ? (unsigned)(slab % slabs_per_sample) * TN : 0u;
+        const unsigned pos = p0 + j;
+        const bool valid = slab_ok && pos < P.outV;
+        const unsigned posc = valid ? pos : P.outV - 1;
+
+        int o[ND], ib[ND];
+        decode_pos<ND>(P, posc, o);
+#pragma unroll
+        for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
+        TapGeo<T, ND> t;
+        tap_setup<T, ND>(P, off + (((size_t)n * P.DG + dg) * P.kV + tap) * ND * P.outV, posc, ib, kd, t);
+        const bool live = valid && t.inside;
+
+        __syncthreads();        // previous slab's MFMA reads are done before LDS is overwritten
+        // grad_output slab: rows m_base .. m_base + MT*TN, lanes along positions (coalesced)
+        const T* gb = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV + posc;
+        for (int mr = q; mr < MT * TN; mr += KL) {
+            const int m = m_base + mr;
+            sA[mr * LD + j] = (valid && m < P.M) ? gb[(size_t)m * P.outV] : (T)0;
+        }
+        // sampled slab: channel c0 + cr for cr in [0, TN)
+        unsigned voff[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
+        const T* chan = in + ((size_t)n * P.C_in + c0) * P.inV;
+#pragma unroll 2
+        for (int cr = q; cr < TN; cr += KL) {
+            T b = 0;
+            if (live && c0 + cr < ce) b = sample<T, ND>(chan, voff, t.f);
+            sB[cr * LD + j] = b;
+            chan += (size_t)KL * P.inV;
+        }
+        __syncthreads();
+        // D[m][channel] += A[m][pos] * B[pos][channel]; lane (j, q) reads row j, position ks*KL + q
+#pragma unroll 4
+        for (int ks = 0; ks < TN / KL; ++ks) {
+            const int pp = ks * KL + q;
+            const T b = sB[j * LD + pp];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(sA[(mt * TN + j) * LD + pp], b, acc[mt]);
+        }
+    }
+
+    const int c = c0 + j;
+    if (c >= ce) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < MM::NACC; ++r) {
+            const int m = m_base + mt * TN + MM::row(r, q);
+            if (m < P.M)
+                atomic_add(gw + (((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap, acc[mt][r]);
+        }
+}
+
+}  // namespace dcn

@@ -1,0 +1,207 @@
+"""autograd Functions of the deformable convolution, mirroring the reference's
+`ConvOffset3dFunction` (deform3d/deform_conv3d_functions/deform_conv3d_function.py:7-77) and
+`ConvOffset2dFunction` (deform2d_double/deform_conv2d_functions/deform_conv2d_function.py:7-77;
+deform2d/deform_conv2d_functions/deform_conv2d_function.py:7-57 is its float, dilation-1,
+group-1, bias-free subset).
+
+Same call shape: `Fn.apply(inputs, offset, weight, bias=None, stride, padding, dilation,
+channel_per_group=1, group=1)`; same dilation-blind output size; same shape checks and messages
+as the reference's `shape_check` (deform3d/lib/deform_conv3d_cuda.cpp:24-87), raised as
+RuntimeError.  Differences: no column workspace is kept on ctx (the kernels never build one),
+float32 and float64 are served by the same class for both 2-D and 3-D, and gradients that are
+not required come back as None instead of crashing (the reference wraps None in Variable, :76).
+All tensors must live on one MI355X; there is no CPU path.
+"""
+import torch
+from torch.autograd import Function
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _ntuple(v, nd):
+    if isinstance(v, int):
+        return (v,) * nd
+    v = tuple(int(x) for x in v)
+    _check(len(v) == nd, "expected %d values, got %r" % (nd, v))
+    return v
+
+
+def output_size(in_sizes, kernel, stride, padding):
+    """The reference formula, dilation not included (deform3d/lib/deform_conv3d_cuda.cpp:15-17;
+    deform_conv3d_function.py:26-27)."""
+    return tuple((i + 2 * p - k) // s + 1 for i, k, s, p in zip(in_sizes, kernel, stride, padding))
+
+
+_OUT_MSG = {3: ("error output ll", "error outhh", "error outww"), 2: ("error outhh", "error outww")}
+_OFF_MSG = {3: ("off l", "off h", "off w"), 2: ("off h", "off w")}
+
+
+def shape_check(nd, inputs, weight, offset, output_shape, channel_per_group, group, stride, padding):
+    """Python restatement of the reference's shape_check with its messages."""
+    _check(weight.dim() == nd + 2, "kernel dim")
+    _check(inputs.dim() == nd + 2, "input dim")
+    _check(inputs.size(1) == weight.size(1) * group, "input c != kernel c")
+    _check(len(output_shape) == nd + 2, "output dim")
+    _check(output_shape[0] == inputs.size(0), "output b != input b")
+    _check(output_shape[1] == weight.size(0), "ou c != ker c")
+    _check(offset.dim() == nd + 2, "off dim")
+    _check(offset.size(0) == inputs.size(0), "off batch")
+    kV = 1
+    for k in weight.shape[2:]:
+        kV *= k
+    _check(channel_per_group > 0 and inputs.size(1) % channel_per_group == 0, "off channel")
+    _check(offset.size(1) == inputs.size(1) // channel_per_group * nd * kV, "off channel")
+    for a in range(nd):
+        _check(offset.size(2 + a) == output_shape[2 + a], _OFF_MSG[nd][a])
+    want = output_size(inputs.shape[2:], weight.shape[2:], stride, padding)
+    for a in range(nd):
+        _check(inputs.size(2 + a) + 2 * padding[a] - weight.size(2 + a) >= 0 and want[a] == output_shape[2 + a],
+               _OUT_MSG[nd][a])
+    _check(group > 0 and weight.size(0) % group == 0, "ou c != ker c")
+
+
+def _device_check(*tensors):
+    t0 = tensors[0]
+    _check(t0.is_cuda, "deformable convolution runs on the GPU only: tensors must be on a HIP device "
+                       "(there is no CPU path in this package)")
+    _check(t0.dtype in _SUFFIX, "dtype must be float32 or float64")
+    for t in tensors[1:]:
+        if t is None:
+            continue
+        _check(t.device == t0.device, "all tensors must be on the same GPU")
+        _check(t.dtype == t0.dtype, "all tensors must have the same dtype")
+
+
+def _geom(nd, inputs, weight, out_sizes, stride, padding, dilation, channel_per_group, group):
+    return ([inputs.size(0), inputs.size(1), weight.size(0)] + list(inputs.shape[2:]) + list(out_sizes) +
+            list(weight.shape[2:]) + list(padding) + list(stride) + list(dilation) + [channel_per_group, group])
+
+
+def _workspace(inputs, weight, group):
+    L = _lib.load()
+    kV = 1
+    for k in weight.shape[2:]:
+        kV *= k
+    nbytes = L.dcn_workspace_bytes(inputs.element_size(), inputs.size(1), weight.size(0), kV, group)
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=inputs.device), int(nbytes)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group):
+    L = _lib.load()
+    stride, padding, dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
+    _device_check(inputs, offset, weight, bias)
+    _check(inputs.dim() == nd + 2, "input dim")
+    _check(weight.dim() == nd + 2, "kernel dim")
+    outs = output_size(inputs.shape[2:], weight.shape[2:], stride, padding)
+    out_shape = (inputs.size(0), weight.size(0)) + outs
+    shape_check(nd, inputs, weight, offset, out_shape, channel_per_group, group, stride, padding)
+    if bias is not None:
+        _check(bias.dim() == 1 and bias.size(0) == weight.size(0), "bias size")
+    inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
+    output = torch.empty(out_shape, dtype=inputs.dtype, device=inputs.device)
+    ws, ws_bytes = _workspace(inputs, weight, group)
+    fn = getattr(L, "dcn%dd_forward_%s" % (nd, _SUFFIX[inputs.dtype]))
+    with torch.cuda.device(inputs.device):
+        rc = fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(),
+                bias.contiguous().data_ptr() if bias is not None else None, output.data_ptr(),
+                *_geom(nd, inputs, weight, outs, stride, padding, dilation, channel_per_group, group),
+                ws.data_ptr(), ws_bytes, _stream())
+    _lib.check(rc)
+    return output
+
+
+def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation, channel_per_group, group,
+              need_data, need_weight):
+    L = _lib.load()
+    _device_check(inputs, offset, weight, grad_output)
+    outs = tuple(grad_output.shape[2:])
+    shape_check(nd, inputs, weight, offset, tuple(grad_output.shape), channel_per_group, group, stride, padding)
+    inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
+    grad_output = grad_output.contiguous()
+    geom = _geom(nd, inputs, weight, outs, stride, padding, dilation, channel_per_group, group)
+    suf = _SUFFIX[inputs.dtype]
+    grad_input = grad_offset = grad_weight = None
+    with torch.cuda.device(inputs.device):
+        if need_data:
+            # the kernels accumulate into grad_input (as the reference's atomicAdd does) and store
+            # every element of grad_offset
+            grad_input = torch.zeros_like(inputs)
+            grad_offset = torch.empty_like(offset)
+            ws, ws_bytes = _workspace(inputs, weight, group)
+            fn = getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))
+            _lib.check(fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
+                          grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, _stream()))
+        if need_weight:
+            grad_weight = torch.zeros_like(weight)          # beta = 1 accumulation, as in the reference
+            fn = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
+            _lib.check(fn(inputs.data_ptr(), offset.data_ptr(), grad_output.data_ptr(), grad_weight.data_ptr(),
+                          *geom, None, 0, _stream()))
+    return grad_input, grad_offset, grad_weight
+
+
+class _ConvOffsetNdFunction(Function):
+    ND = 0
+
+    @classmethod
+    def _fwd(cls, ctx, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group):
+        nd = cls.ND
+        ctx.stride, ctx.padding, ctx.dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
+        ctx.channel_per_group, ctx.group = int(channel_per_group), int(group)
+        ctx.has_bias = bias is not None
+        ctx.save_for_backward(inputs, offset, weight)
+        return _forward(nd, inputs, offset, weight, bias, ctx.stride, ctx.padding, ctx.dilation,
+                        ctx.channel_per_group, ctx.group)
+
+    @classmethod
+    def _bwd(cls, ctx, grad_output):
+        inputs, offset, weight = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        # grad_input and grad_offset come out of one kernel, as in the reference (:52)
+        gi, go, gw = _backward(cls.ND, inputs, offset, weight, grad_output, ctx.stride, ctx.padding, ctx.dilation,
+                               ctx.channel_per_group, ctx.group, need[0] or need[1], need[2])
+        gb = None
+        if ctx.has_bias and need[3]:
+            gb = grad_output.sum(dim=[0] + list(range(2, 2 + cls.ND)))
+        return (gi if need[0] else None, go if need[1] else None, gw, gb, None, None, None, None, None)
+
+
+class ConvOffset3dFunction(_ConvOffsetNdFunction):
+    ND = 3
+
+    @staticmethod
+    def forward(ctx, inputs, offset, weight, bias=None, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
+                channel_per_group=1, group=1):
+        return ConvOffset3dFunction._fwd(ctx, inputs, offset, weight, bias, stride, padding, dilation,
+                                         channel_per_group, group)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        return ConvOffset3dFunction._bwd(ctx, grad_output)
+
+
+class ConvOffset2dFunction(_ConvOffsetNdFunction):
+    ND = 2
+
+    @staticmethod
+    def forward(ctx, inputs, offset, weight, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
+                channel_per_group=1, group=1):
+        return ConvOffset2dFunction._fwd(ctx, inputs, offset, weight, bias, stride, padding, dilation,
+                                         channel_per_group, group)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        return ConvOffset2dFunction._bwd(ctx, grad_output)

@@ -1,0 +1,69 @@
+"""nn.Module front ends, mirroring `ConvOffset3d`
+(deform3d/deform_conv3d_modules/deform_conv3d_model.py:11-50) and `ConvOffset2d`
+(deform2d_double/deform_conv2d_modules/deform_conv2d_model.py:11-50).
+
+Constructor: `(in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+channel_per_group=1, bias=True, groups=1)`, forward `(input, offset)`; parameters are named
+`weight` [out, in/groups, *kernel] and `bias` [out], so state_dicts interchange.  The legacy
+float 2-D module (deform2d/deform_conv2d_modules/deform_conv2d_model.py:12-18) takes
+`channel_per_group` as its 6th positional argument; here that slot is `dilation` as in the other
+two packages, so pass `channel_per_group` by keyword.
+
+Initialisation: the reference draws Kaiming-normal (fan_out) and then overwrites the weight with
+the constant 1 (deform_conv3d_model.py:38-39); this keeps the Kaiming draw, which is what the
+float 2-D package does (deform2d ... :29).  Bias ~ U(-0.1, 0.1) as in the reference (:42).
+`device` and `dtype` are extra keyword arguments (the reference hard-codes cuda float / double).
+"""
+import torch
+import torch.nn as nn
+from torch.nn.modules.utils import _pair, _triple
+
+from .functions import ConvOffset2dFunction, ConvOffset3dFunction
+
+
+class _ConvOffsetNd(nn.Module):
+    _tuple = None
+    _function = None
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 channel_per_group=1, bias=True, groups=1, device=None, dtype=None):
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.kernel_size = self._tuple(kernel_size)
+        self.stride = self._tuple(stride)
+        self.padding = self._tuple(padding)
+        self.dilation = self._tuple(dilation)
+        self.channel_per_group = channel_per_group
+        self.group = groups
+        if in_channels % groups != 0:
+            raise ValueError('in_channels must be divisible by groups')
+        if out_channels % groups != 0:
+            raise ValueError('out_channels must be divisible by groups')
+        kw = dict(device=device, dtype=dtype)
+        self.weight = nn.Parameter(torch.empty(out_channels, in_channels // groups, *self.kernel_size, **kw))
+        nn.init.kaiming_normal_(self.weight, mode='fan_out')
+        if bias:
+            self.bias = nn.Parameter(torch.empty(out_channels, **kw))
+            nn.init.uniform_(self.bias, -0.1, 0.1)
+        else:
+            self.register_parameter('bias', None)
+
+    def forward(self, input, offset):
+        return self._function.apply(input, offset, self.weight, self.bias, self.stride, self.padding,
+                                    self.dilation, self.channel_per_group, self.group)
+
+    def extra_repr(self):
+        return ('{in_channels}, {out_channels}, kernel_size={kernel_size}, stride={stride}, padding={padding}, '
+                'dilation={dilation}, channel_per_group={channel_per_group}, groups={group}, '
+                'bias=' + str(self.bias is not None)).format(**self.__dict__)
+
+
+class ConvOffset3d(_ConvOffsetNd):
+    _tuple = staticmethod(_triple)
+    _function = ConvOffset3dFunction
+
+
+class ConvOffset2d(_ConvOffsetNd):
+    _tuple = staticmethod(_pair)
+    _function = ConvOffset2dFunction

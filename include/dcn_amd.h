@@ -1,0 +1,125 @@
+/*
+ * dcn_amd.h -- C ABI of the MI355X (gfx950) deformable-convolution library, libdcn_amd.so.
+ *
+ * Drop-in boundary for the three native entry points each operator package of
+ * lshiwjx/deform_conv3d_pytorch_op binds through cffi:
+ *
+ *   deform_conv_forward_cuda                 deform3d/lib/deform_conv3d_cuda.h:12-18
+ *                                            deform2d_double/lib/deform_conv2d_cuda.h:12-18
+ *                                            deform2d/lib/deform_conv2d_cuda.h:12-17
+ *   deform_conv_backward_input_offset_cuda   deform3d/lib/deform_conv3d_cuda.h:20-26
+ *                                            deform2d_double/lib/deform_conv2d_cuda.h:20-26
+ *                                            deform2d/lib/deform_conv2d_cuda.h:19-24
+ *   deform_conv_backward_weight_cuda         deform3d/lib/deform_conv3d_cuda.h:28-34
+ *                                            deform2d_double/lib/deform_conv2d_cuda.h:28-34
+ *                                            deform2d/lib/deform_conv2d_cuda.h:26-31
+ *
+ * The reference passes THCudaTensor handles; here every tensor is a raw device pointer to a
+ * contiguous row-major buffer and every extent is an explicit int, in the reference's argument
+ * order (pad, stride, dilation triples, channel_per_deformable_group, group).  Layouts:
+ *
+ *   input        [batch][input_c][input_l][input_h][input_w]              (no input_l in 2-D)
+ *   weight       [output_c][input_c / group][kernel_l][kernel_h][kernel_w]
+ *   offset       [batch][input_c / channel_per_deformable_group][kernel volume][nd][output volume]
+ *                axis order (l, h, w) in 3-D and (h, w) in 2-D
+ *   output       [batch][output_c][output_l][output_h][output_w]
+ *
+ * Differences from the reference ABI, all on purpose:
+ *   - there is no `columns` argument: the sampled column buffer never exists in device memory;
+ *   - `workspace` is caller-owned scratch of at least dcn_workspace_bytes(...) bytes (it holds a
+ *     re-laid-out copy of the weights); the library never allocates device memory;
+ *   - `stream` is the hipStream_t to enqueue on (NULL = the null stream); calls are asynchronous;
+ *   - the return value is 0 on success and a negative DCN_E_* code on failure, with the text
+ *     from dcn_last_error() (thread-local).  The reference returns 1 and raises through THError.
+ *   - the caller's weight tensor is never reshaped in place (the reference does that).
+ *
+ * Caller obligations kept from the reference: `output` and `grad_offset` are fully overwritten;
+ * `grad_input` and `grad_weight` are ACCUMULATED into and must be zero-filled by the caller when
+ * a plain gradient is wanted (deform3d/deform_conv3d_functions/deform_conv3d_function.py:53,64).
+ * Output extents must satisfy the reference formula out = (in + 2*pad - kernel) / stride + 1
+ * (integer division, dilation not included; deform3d/lib/deform_conv3d_cuda.cpp:15-17,81-86).
+ */
+#ifndef DCN_AMD_H
+#define DCN_AMD_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DCN_OK            0
+#define DCN_E_ARGUMENT   -1   /* inconsistent extents, null pointer, unsupported size */
+#define DCN_E_WORKSPACE  -2   /* workspace missing or too small */
+#define DCN_E_LAUNCH     -3   /* HIP reported an error when launching */
+#define DCN_E_DEVICE     -4   /* current device is not a gfx950 GPU */
+
+int dcn_version(void);              /* ABI version, currently 1 */
+const char *dcn_arch(void);         /* the code-object target the kernels were built for: "gfx950" */
+const char *dcn_last_error(void);   /* message of the last failing call on this thread ("" if none) */
+
+/* Scratch bytes any of the three calls below needs for this layer (elem_size 4 = f32, 8 = f64). */
+size_t dcn_workspace_bytes(int elem_size, int input_c, int output_c, int kernel_volume, int group);
+
+/* ---- 3-D, trilinear ------------------------------------------------------------------------
+ * replaces deform3d/lib/deform_conv3d_cuda.cpp:90-165 (forward), :168-262 (backward_input_offset)
+ * and :265-336 (backward_weight).  The reference instantiates float only; f64 is the same
+ * arithmetic in double.  `bias` ([output_c] or NULL) is added in the epilogue; the reference adds
+ * it from Python (deform_conv3d_function.py:41-42). */
+#define DCN3D_GEOMETRY                                                                           \
+    int batch, int input_c, int output_c, int input_l, int input_h, int input_w, int output_l,   \
+    int output_h, int output_w, int kernel_l, int kernel_h, int kernel_w, int pad_l, int pad_h,  \
+    int pad_w, int stride_l, int stride_h, int stride_w, int dilation_l, int dilation_h,         \
+    int dilation_w, int channel_per_deformable_group, int group
+
+int dcn3d_forward_f32(const float *input, const float *weight, const float *offset, const float *bias,
+                      float *output, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn3d_forward_f64(const double *input, const double *weight, const double *offset, const double *bias,
+                      double *output, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+
+int dcn3d_backward_input_offset_f32(const float *input, const float *weight, const float *offset,
+                                    const float *grad_output, float *grad_input, float *grad_offset,
+                                    DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn3d_backward_input_offset_f64(const double *input, const double *weight, const double *offset,
+                                    const double *grad_output, double *grad_input, double *grad_offset,
+                                    DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+
+int dcn3d_backward_weight_f32(const float *input, const float *offset, const float *grad_output,
+                              float *grad_weight, DCN3D_GEOMETRY, void *workspace,
+                              size_t workspace_bytes, void *stream);
+int dcn3d_backward_weight_f64(const double *input, const double *offset, const double *grad_output,
+                              double *grad_weight, DCN3D_GEOMETRY, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
+/* ---- 2-D, bilinear -------------------------------------------------------------------------
+ * replaces deform2d_double/lib/deform_conv2d_cuda.cpp:82-155, :158-249, :252-325 (double, with
+ * dilation and groups) and deform2d/lib/deform_conv2d_cuda.cpp:82-128, :131-190, :193-235
+ * (float; its ABI has no dilation/group arguments: pass dilation 1, group 1). */
+#define DCN2D_GEOMETRY                                                                           \
+    int batch, int input_c, int output_c, int input_h, int input_w, int output_h, int output_w,  \
+    int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,                \
+    int dilation_h, int dilation_w, int channel_per_deformable_group, int group
+
+int dcn2d_forward_f32(const float *input, const float *weight, const float *offset, const float *bias,
+                      float *output, DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn2d_forward_f64(const double *input, const double *weight, const double *offset, const double *bias,
+                      double *output, DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+
+int dcn2d_backward_input_offset_f32(const float *input, const float *weight, const float *offset,
+                                    const float *grad_output, float *grad_input, float *grad_offset,
+                                    DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn2d_backward_input_offset_f64(const double *input, const double *weight, const double *offset,
+                                    const double *grad_output, double *grad_input, double *grad_offset,
+                                    DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+
+int dcn2d_backward_weight_f32(const float *input, const float *offset, const float *grad_output,
+                              float *grad_weight, DCN2D_GEOMETRY, void *workspace,
+                              size_t workspace_bytes, void *stream);
+int dcn2d_backward_weight_f64(const double *input, const double *offset, const double *grad_output,
+                              double *grad_weight, DCN2D_GEOMETRY, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DCN_AMD_H */

@@ -1,0 +1,56 @@
+"""Seeded problem instances shared by the CPU and GPU tests."""
+import math
+
+import torch
+
+
+def _t(v, nd):
+    return (v,) * nd if isinstance(v, int) else tuple(v)
+
+
+def output_size(ins, ks, stride, pad):
+    return tuple((i + 2 * p - k) // s + 1 for i, k, s, p in zip(ins, ks, stride, pad))
+
+
+def make_case(nd, N, C_in, C_out, ins, k, stride, pad, dil, cpg, groups, off_scale, dtype=torch.float64,
+              seed=0, bias=True, off_dist="uniform"):
+    g = torch.Generator().manual_seed(seed)
+    ins, k, stride, pad, dil = _t(ins, nd), _t(k, nd), _t(stride, nd), _t(pad, nd), _t(dil, nd)
+    outs = output_size(ins, k, stride, pad)
+    kV = math.prod(k)
+    x = torch.randn((N, C_in) + ins, generator=g, dtype=torch.float64)
+    oshape = (N, C_in // cpg * nd * kV) + outs
+    if off_dist == "uniform":
+        off = (torch.rand(oshape, generator=g, dtype=torch.float64) * 2 - 1) * off_scale
+    else:   # N(0,1) with 10 % of the entries replaced by U[-6,6]  (BASELINE configs[2])
+        off = torch.randn(oshape, generator=g, dtype=torch.float64)
+        mask = torch.rand(oshape, generator=g, dtype=torch.float64) < 0.1
+        wide = (torch.rand(oshape, generator=g, dtype=torch.float64) * 2 - 1) * 6
+        off = torch.where(mask, wide, off)
+    fan_out = C_out * kV
+    w = torch.randn((C_out, C_in // groups) + k, generator=g, dtype=torch.float64) * math.sqrt(2.0 / fan_out)
+    b = torch.randn(C_out, generator=g, dtype=torch.float64) if bias else None
+    gout = torch.randn((N, C_out) + outs, generator=g, dtype=torch.float64)
+    cast = lambda t: None if t is None else t.to(dtype).contiguous()
+    return dict(x=cast(x), off=cast(off), w=cast(w), b=cast(b), gout=cast(gout), stride=stride, pad=pad, dil=dil,
+                cpg=cpg, groups=groups, ins=ins, k=k, outs=outs, nd=nd)
+
+
+# nd, N, Cin, Cout, in, k, stride, pad, dil, cpg, groups, off_scale
+SMALL_CASES = {
+    "2d_basic": (2, 2, 4, 6, (7, 9), 3, 1, 1, 1, 2, 2, 3.0),
+    "2d_rect_kernel_stride_dil": (2, 1, 6, 4, (8, 6), (3, 2), (2, 1), (2, 1), (2, 1), 3, 1, 2.0),
+    "2d_ref_gradient_script": (2, 2, 2, 4, 7, 1, 2, 2, 2, 2, 2, 1.0),      # deform2d_double/test_gradient.py:7-19
+    "2d_c1": (2, 2, 8, 8, 16, 3, 1, 1, 1, 8, 1, 1.5),                     # BASELINE configs[0]
+    "2d_wide_m": (2, 1, 40, 72, (9, 11), 3, 1, 1, 1, 20, 1, 2.0),          # several MFMA row tiles, 2 deformable groups
+    "2d_many_m_chunks": (2, 1, 6, 300, (6, 7), 3, 1, 1, 1, 6, 1, 1.0),     # M > 8 row tiles of 32
+    "2d_c3_like": (2, 1, 16, 8, 10, 3, 1, 2, 2, 4, 2, 3.0),                # groups 2, 4 deformable groups, dilation 2
+    "2d_cpg_straddles_groups": (2, 1, 12, 4, 6, 3, 1, 1, 1, 12, 2, 1.5),   # one deformable group over two conv groups
+    "2d_cpg_unaligned": (2, 1, 12, 6, 6, 2, 1, 0, 1, 4, 2, 1.5),           # cpg 4, 6 channels per conv group
+    "3d_basic": (3, 2, 4, 4, (5, 6, 7), 3, 1, 1, 1, 2, 2, 3.0),
+    "3d_mixed": (3, 1, 6, 3, (4, 7, 5), (2, 3, 1), (1, 2, 1), (1, 2, 0), (1, 2, 1), 2, 3, 2.0),
+    "3d_ref_gradient_script": (3, 2, 2, 4, 7, 3, 2, 2, 2, 2, 2, 1.0),      # deform3d/test_gradient.py:9-20
+    "3d_c4_like": (3, 2, 40, 40, (4, 9, 10), 3, 1, 1, 1, 40, 1, 1.5),      # one deformable group, >1 channel tile
+    "3d_c5_like": (3, 1, 16, 24, (4, 12, 12), 3, (1, 2, 2), 1, 1, 4, 1, 2.0),   # strided, 4 deformable groups
+    "3d_short_length": (3, 1, 4, 4, (2, 8, 8), (1, 3, 3), 1, (0, 1, 1), 1, 4, 1, 4.0),  # D < H: out-of-range branch vs length extent
+}
