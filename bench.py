@@ -124,7 +124,8 @@ def main():
     L = _lib.load()
     suf = "f32" if dtype == torch.float32 else "f64"
     geom = _geom(nd, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
-    nbytes = L.dcn_workspace_bytes(x.element_size(), x.shape[1], w.shape[0], math.prod(c["k"]), c["groups"])
+    nbytes = L.dcn_workspace_bytes(x.element_size(), x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]),
+                                   math.prod(c["k"]), c["groups"])
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     out = torch.empty((x.shape[0], w.shape[0]) + c["outs"], dtype=dtype, device=dev)
     gin, goff, gw = torch.zeros_like(x), torch.empty_like(off), torch.zeros_like(w)

@@ -29,17 +29,25 @@ template <typename T> void fwd_weight_pad(int M, int Cg, int& MT, int& mchunks, 
     Mp = mchunks * MT * TN;
     Cgp = Cg + KL;
 }
-template <typename T> void bwd_weight_pad(int M, int Cg, int& Mp, int& Cgp) {
+template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp) {
     Mp = M + Mma<T>::KL;
     Cgp = Cg + Mma<T>::TN;
 }
-template <typename T> size_t workspace_need(int C_in, int C_out, int kV, int G) {
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+// Workspace of backward_input_offset: [ re-laid-out weight | input channels-last | grad-input channels-last ]
+template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G) {
+    int Mp, Cgp;
+    bwd_data_weight_pad<T>(M, Cg, Mp, Cgp);
+    return align256((size_t)G * kV * Mp * Cgp * sizeof(T));
+}
+template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, int kV, int G) {
     const int M = C_out / G, Cg = C_in / G;
-    int MT, mchunks, Mp, Cgp, Mp2, Cgp2;
+    int MT, mchunks, Mp, Cgp;
     fwd_weight_pad<T>(M, Cg, MT, mchunks, Mp, Cgp);
-    bwd_weight_pad<T>(M, Cg, Mp2, Cgp2);
-    const size_t a = (size_t)G * kV * Mp * Cgp, b = (size_t)G * kV * Mp2 * Cgp2;
-    return (a > b ? a : b) * sizeof(T);
+    const size_t fwd = (size_t)G * kV * Mp * Cgp * sizeof(T);
+    const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
+    return fwd > bwd ? fwd : bwd;
 }
 
 struct Geometry {   // the reference's argument list, 2-D mapped onto slots 1,2 with a unit length axis
@@ -64,6 +72,9 @@ int validate(const Geometry& g, Params& P) {
     const long long inV = (long long)g.in[0] * g.in[1] * g.in[2], outV = (long long)g.out[0] * g.out[1] * g.out[2];
     // per-channel offsets are 32-bit inside the kernels (including a bias of up to 4 channels)
     if (inV > (1ll << 27) || outV > (1ll << 27)) return fail(DCN_E_ARGUMENT, "a single channel exceeds 2^27 voxels");
+    // channels-last voxel*channel offsets of one sample are 32-bit as well
+    if (inV * g.C_in > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one input sample exceeds 2^31 elements");
+    if (g.N > 65535) return fail(DCN_E_ARGUMENT, "batch exceeds 65535");
     P.nd = g.nd; P.N = g.N; P.C_in = g.C_in; P.C_out = g.C_out; P.G = g.G; P.cpg = g.cpg; P.DG = g.C_in / g.cpg;
     P.M = g.C_out / g.G; P.Cg = g.C_in / g.G;
     for (int a = 0; a < 3; ++a) {
@@ -122,15 +133,28 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
-    bwd_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
-    if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
+    bwd_data_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
+    const size_t wbytes = bwd_data_weight_bytes<T>(P.M, P.Cg, P.kV, P.G);
+    const size_t tbytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
+    if (!ws || ws_bytes < wbytes + 2 * tbytes) return fail(DCN_E_WORKSPACE, "workspace too small");
     T* wt = static_cast<T*>(ws);
+    T* in_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes);
+    T* gin_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes + tbytes);
     if (int rc = relayout<T>(P, w, wt, 1, s)) return rc;
+    const dim3 tgrid((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N), tblock(32, 8);
+    hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
+    if (int rc = check_launch("to_channels_last_kernel")) return rc;
+    const size_t nelem = (size_t)P.N * P.C_in * P.inV;
+    const unsigned fblocks = (unsigned)((nelem + 1023) / 1024 > 8192 ? 8192 : (nelem + 1023) / 1024);
+    hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fblocks), dim3(256), 0, s, gin_cl, nelem);
+    if (int rc = check_launch("fill_zero_kernel")) return rc;
     const int TN = Mma<T>::TN;
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
-    hipLaunchKernelGGL((backward_data_kernel<T, ND>), grid, dim3(WG), 0, s, P, in, off, wt, gout, gin, goff);
-    return check_launch("backward_data_kernel");
+    hipLaunchKernelGGL((backward_data_kernel<T, ND>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff);
+    if (int rc = check_launch("backward_data_kernel")) return rc;
+    hipLaunchKernelGGL(add_from_channels_last_kernel<T>, tgrid, tblock, 0, s, gin_cl, gin, P.C_in, P.inV);
+    return check_launch("add_from_channels_last_kernel");
 }
 
 template <typename T, int ND, int MT>
@@ -216,10 +240,11 @@ int dcn_version(void) { return 1; }
 const char* dcn_arch(void) { return "gfx950"; }
 const char* dcn_last_error(void) { return g_err.c_str(); }
 
-size_t dcn_workspace_bytes(int elem_size, int input_c, int output_c, int kernel_volume, int group) {
-    if (group <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0) return 0;
-    return elem_size == 8 ? workspace_need<double>(input_c, output_c, kernel_volume, group)
-                          : workspace_need<float>(input_c, output_c, kernel_volume, group);
+size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
+                           int kernel_volume, int group) {
+    if (group <= 0 || batch <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0 || input_volume == 0) return 0;
+    return elem_size == 8 ? workspace_need<double>(batch, input_c, output_c, input_volume, kernel_volume, group)
+                          : workspace_need<float>(batch, input_c, output_c, input_volume, kernel_volume, group);
 }
 
 #define DEFINE_OPS(SUF, T)                                                                                          \

@@ -67,7 +67,7 @@ template <int ND> __device__ inline constexpr int slot(int a) { return a + 3 - N
 
 template <int ND>
 __device__ inline void decode_pos(const Params& P, unsigned pos, int o[ND]) {
-    if (ND == 3) {
+    if constexpr (ND == 3) {
         o[2] = pos % P.out[2];
         unsigned t = pos / P.out[2];
         o[1] = t % P.out[1];
@@ -80,7 +80,7 @@ __device__ inline void decode_pos(const Params& P, unsigned pos, int o[ND]) {
 
 template <int ND>
 __device__ inline void decode_tap(const Params& P, int tap, int kk[ND]) {
-    if (ND == 3) {
+    if constexpr (ND == 3) {
         kk[2] = tap % P.k[2];
         int t = tap / P.k[2];
         kk[1] = t % P.k[1];
@@ -122,7 +122,7 @@ __device__ inline void tap_setup(const Params& P, const T* __restrict__ off_tap,
         t.f[a] = p - (T)l;
     }
     t.inside = inside;
-    if (ND == 3) {
+    if constexpr (ND == 3) {
         const unsigned s1 = P.in[2], s2 = P.in[1] * P.in[2];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
@@ -144,7 +144,7 @@ __device__ inline void tap_setup(const Params& P, const T* __restrict__ off_tap,
 // first voxel; `voff` are the corner offsets (possibly biased by the caller, see kernels).
 template <typename T, int ND>
 __device__ inline T sample(const T* __restrict__ chan, const unsigned* voff, const T* f) {
-    if (ND == 3) {
+    if constexpr (ND == 3) {
         const T c000 = chan[voff[0]], c001 = chan[voff[1]], c010 = chan[voff[2]], c011 = chan[voff[3]];
         const T c100 = chan[voff[4]], c101 = chan[voff[5]], c110 = chan[voff[6]], c111 = chan[voff[7]];
         const T fw = f[2], gw = (T)1 - fw, fh = f[1], gh = (T)1 - fh, fl = f[0], gl = (T)1 - fl;

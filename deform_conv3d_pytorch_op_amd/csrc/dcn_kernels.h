@@ -112,30 +112,115 @@ __global__ __launch_bounds__(WG) void forward_kernel(Params P, const T* __restri
 }
 
 // ---------------------------------------------------------------------------------------------
-// Backward to input and offset.  Per (tap, TN channels, TN positions) the grad-column tile
-//     gcol[c][pos] = sum_m W[g*M+m][c][tap] * gout[n][g*M+m][pos]
+// Layout changes between [C][V] (channel planes, what PyTorch hands over) and [V][C]
+// (channels-last, what the scatter / coordinate kernel wants so that the lanes of a wavefront
+// touch consecutive addresses).  32x32 tiles through LDS; grid (ceil(V/32), ceil(C/32), N),
+// block (32, 8).
+template <typename T>
+__global__ void to_channels_last_kernel(const T* __restrict__ src, T* __restrict__ dst, int C, unsigned V) {
+    __shared__ T tile[32][33];
+    const size_t base = (size_t)blockIdx.z * C * V;
+    const unsigned v0 = blockIdx.x * 32;
+    const int c0 = blockIdx.y * 32;
+    for (int i = threadIdx.y; i < 32; i += 8) {
+        const int c = c0 + i;
+        const unsigned v = v0 + threadIdx.x;
+        if (c < C && v < V) tile[i][threadIdx.x] = src[base + (size_t)c * V + v];
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += 8) {
+        const unsigned v = v0 + i;
+        const int c = c0 + threadIdx.x;
+        if (c < C && v < V) dst[base + (size_t)v * C + c] = tile[threadIdx.x][i];
+    }
+}
+
+// dst[C][V] += src[V][C]
+template <typename T>
+__global__ void add_from_channels_last_kernel(const T* __restrict__ src, T* __restrict__ dst, int C, unsigned V) {
+    __shared__ T tile[32][33];
+    const size_t base = (size_t)blockIdx.z * C * V;
+    const unsigned v0 = blockIdx.x * 32;
+    const int c0 = blockIdx.y * 32;
+    for (int i = threadIdx.y; i < 32; i += 8) {
+        const unsigned v = v0 + i;
+        const int c = c0 + threadIdx.x;
+        if (c < C && v < V) tile[i][threadIdx.x] = src[base + (size_t)v * C + c];
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += 8) {
+        const int c = c0 + i;
+        const unsigned v = v0 + threadIdx.x;
+        if (c < C && v < V) dst[base + (size_t)c * V + v] += tile[threadIdx.x][i];
+    }
+}
+
+template <typename T>
+__global__ void fill_zero_kernel(T* __restrict__ p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+// Sum over the TN lanes that share a reduction slot (lanes l with equal l / TN).  For float the
+// 16-lane rows are summed with DPP adds and the two rows of a 32-lane group are joined with a
+// row broadcast, so the result is only guaranteed in the UPPER 16 lanes of each group; for
+// double a shuffle butterfly leaves it in every lane.  holder(j) tells which lanes hold it.
+template <int CTRL, int ROW_MASK>
+__device__ inline float dpp_term(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+__device__ inline float group_sum(float v) {
+    v += dpp_term<0xB1, 0xF>(v);      // quad_perm [1,0,3,2]
+    v += dpp_term<0x4E, 0xF>(v);      // quad_perm [2,3,0,1]
+    v += dpp_term<0x141, 0xF>(v);     // row_half_mirror
+    v += dpp_term<0x140, 0xF>(v);     // row_mirror: every lane of a 16-lane row holds the row sum
+    v += dpp_term<0x142, 0xA>(v);     // row_bcast15 into rows 1 and 3: upper row of each 32-lane group
+    return v;
+}
+__device__ inline double group_sum(double v) {
+#pragma unroll
+    for (int sh = 1; sh < 16; sh <<= 1) v += __shfl_xor(v, sh);
+    return v;
+}
+template <typename T> __device__ inline bool sum_holder(int j);
+template <> __device__ inline bool sum_holder<float>(int j) { return j >= 16; }
+template <> __device__ inline bool sum_holder<double>(int) { return true; }
+
+// ---------------------------------------------------------------------------------------------
+// Backward to input and offset, channels-last.  Per (tap, TN positions, TN channels) the
+// transposed grad-column tile
+//     gcolT[pos][c] = sum_m gout[n][g*M+m][pos] * W[g*M+m][c][tap]
 // is formed by MFMA (replaces the Sgemm at deform3d/lib/deform_conv3d_cuda.cpp:213-220) and lands
-// with lane = position, registers = channels, which is exactly what the two consumers need:
+// with lanes along CHANNELS and registers along positions.  With input and grad-input held
+// channels-last ([voxel][channel]) every corner access of the two consumers is one contiguous
+// run of TN channels per lane group:
 //   col2im_input  (deform3d kernel.cu:229-296, 2-D deform2d_double kernel.cu:201-238): the value
-//                 is scattered to the 8 (4) corners with weights (w_l*w_h*w_w)*gcol;
+//                 is added to the 8 (4) corners with weights (w_l*w_h*w_w)*gcol by hardware float
+//                 atomics on consecutive addresses;
 //   col2im_offset (deform3d kernel.cu:386-483, 2-D :309-366): gcol times the derivative of the
-//                 interpolation along each axis, summed over the channels of the deformable group,
-//                 plus -- 3-D only -- the out-of-range branches (:470-481), which compare the h
-//                 and w coordinates against the LENGTH extent exactly like the reference.
+//                 interpolation along each axis, summed over the channels of the deformable
+//                 group -- a reduction across lanes -- plus, 3-D only, the out-of-range branches
+//                 (:470-481), which compare the h and w coordinates against the LENGTH extent
+//                 exactly like the reference.
+// The geometry of a (tap, position) is computed once by the lane that owns the position and
+// handed to the channel lanes through LDS.
 // grid.x = N * tiles, grid.y = DG.  grad_offset gets a plain store of every element.
 template <typename T, int ND>
-__global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __restrict__ in,
+__global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __restrict__ in_cl,
                                                            const T* __restrict__ off, const T* __restrict__ Wt,
-                                                           const T* __restrict__ gout, T* __restrict__ gin,
+                                                           const T* __restrict__ gout, T* __restrict__ gin_cl,
                                                            T* __restrict__ goff) {
     using MM = Mma<T>;
-    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
+    __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // corner voxel index * C_in
+    __shared__ __align__(16) T sCw[WAVES][TN][NC];           // corner weights
+    __shared__ __align__(16) T sMisc[WAVES][TN][8];          // f[ND] | oob sign[ND] at 3.. | inside flag at 6
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     const int n = blockIdx.x / P.tiles, tile = blockIdx.x % P.tiles;
     const int dg = blockIdx.y;
 
-    const unsigned pos = (unsigned)(tile * WAVES + wave) * TN + j;
+    const unsigned pos0 = (unsigned)(tile * WAVES + wave) * TN;
+    const unsigned pos = pos0 + j;
     const bool valid = pos < P.outV;
     const unsigned posc = valid ? pos : P.outV - 1;
     int o[ND], ib[ND];
@@ -146,6 +231,8 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
     T* goff_dg = goff + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+    const T* in_n = in_cl + (size_t)n * P.inV * P.C_in;
+    T* gin_n = gin_cl + (size_t)n * P.inV * P.C_in;
 
     for (int tap = 0; tap < P.kV; ++tap) {
         int kk[ND], kd[ND];
@@ -155,90 +242,116 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
         TapGeo<T, ND> t;
         tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, posc, ib, kd, t);
         const bool live = valid && t.inside;
-
-        // corner weights, multiplied in the reference's order (w_l * w_h * w_w)
-        T cw[NC];
-        if (ND == 3) {
-            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
-            cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
-            cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
-        } else {
-            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-            cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
-        }
-        // 3-D out-of-range branches: sign per axis for |gcol| (0 = no contribution)
-        T oob[ND];
-#pragma unroll
-        for (int a = 0; a < ND; ++a) oob[a] = 0;
+        T oob[3] = {0, 0, 0};
         if (ND == 3 && valid && !t.inside) {
             const T len = (T)P.in[0];
 #pragma unroll
-            for (int a = 0; a < 3; ++a) oob[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= len) ? (T)1 : (T)0);
+            for (int a = 0; a < ND; ++a) oob[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= len) ? (T)1 : (T)0);
         }
-        const bool any_oob = (ND == 3) && (oob[0] != 0 || oob[ND - 2] != 0 || oob[ND - 1] != 0);
-        T ga[ND];
-#pragma unroll
-        for (int a = 0; a < ND; ++a) ga[a] = 0;
+        const bool any_oob = oob[0] != 0 || oob[1] != 0 || oob[2] != 0;
+        const bool work = __any(live || any_oob);
 
-        if (__any(live || any_oob)) {
+        __syncthreads();            // the previous tap's readers are done
+        if (q == 0) {
+            T cw[NC];
+            if constexpr (ND == 3) {   // multiplied in the reference's order (w_l * w_h * w_w)
+                const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+            } else {
+                const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+            }
+#pragma unroll
+            for (int i = 0; i < NC; ++i) {
+                sIdx[wave][j][i] = t.idx[i] * (unsigned)P.C_in;
+                sCw[wave][j][i] = cw[i];
+            }
+#pragma unroll
+            for (int a = 0; a < ND; ++a) sMisc[wave][j][a] = t.f[a];
+#pragma unroll
+            for (int a = 0; a < 3; ++a) sMisc[wave][j][3 + a] = oob[a];
+            sMisc[wave][j][6] = live ? (T)1 : (T)0;
+        }
+        __syncthreads();
+
+        T ga[NACC][ND];
+#pragma unroll
+        for (int r = 0; r < NACC; ++r)
+#pragma unroll
+            for (int a = 0; a < ND; ++a) ga[r][a] = 0;
+
+        if (work) {
             for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
                 const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
                 const T* gb = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV + posc;
                 for (int c0 = rb; c0 < re; c0 += TN) {
                     typename MM::Acc d = acc_zero<T>();
-                    const T* wa = Wt + (((size_t)g * P.kV + tap) * P.Mp + q) * P.Cgp + (c0 - g * P.Cg) + j;
+                    const T* wb = Wt + (((size_t)g * P.kV + tap) * P.Mp + q) * P.Cgp + (c0 - g * P.Cg) + j;
                     const T* gq = gb + (size_t)q * P.outV;
                     for (int m0 = 0; m0 < P.M; m0 += KL) {
-                        const T a = *wa;
-                        const T b = (valid && m0 + q < P.M) ? *gq : (T)0;
+                        const T a = (valid && m0 + q < P.M) ? *gq : (T)0;      // A[row = position j][k = m]
+                        const T b = *wb;                                       // B[k = m][col = channel j]
                         d = MM::mma(a, b, d);
-                        wa += (size_t)KL * P.Cgp;
+                        wb += (size_t)KL * P.Cgp;
                         gq += (size_t)KL * P.outV;
                     }
+                    const int c = c0 + j;
+                    if (c < re) {
 #pragma unroll
-                    for (int r = 0; r < MM::NACC; ++r) {
-                        const int c = c0 + MM::row(r, q);
-                        if (c >= re) continue;
-                        const T gv = d[r];
-                        if (live) {
-                            const T* ic = in + ((size_t)n * P.C_in + c) * P.inV;
-                            T* gc = gin + ((size_t)n * P.C_in + c) * P.inV;
-                            T v[NC];
+                        for (int r = 0; r < NACC; ++r) {
+                            const int rho = MM::row(r, q);
+                            const T gv = d[r];
+                            const T* misc = sMisc[wave][rho];
+                            if (misc[6] != (T)0) {
+                                unsigned ix[NC];
+                                T v[NC];
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
-                            if (ND == 3) {
-                                const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh,
-                                        fw = t.f[2], gw = (T)1 - fw;
-                                const T dl = ((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
-                                             ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh;
-                                const T dh = ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
-                                             ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl;
-                                const T dw = ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
-                                             ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
-                                ga[0] += gv * dl; ga[1] += gv * dh; ga[2] += gv * dw;
-                            } else {
-                                const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                                ga[0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
-                                ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
+                                for (int i = 0; i < NC; ++i) ix[i] = sIdx[wave][rho][i] + (unsigned)c;
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) v[i] = in_n[ix[i]];
+                                if constexpr (ND == 3) {
+                                    const T fl = misc[0], gl = (T)1 - fl, fh = misc[1], gh = (T)1 - fh,
+                                            fw = misc[2], gw = (T)1 - fw;
+                                    const T dl = ((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
+                                                 ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh;
+                                    const T dh = ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
+                                                 ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl;
+                                    const T dw = ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                                 ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
+                                    ga[r][0] += gv * dl; ga[r][1] += gv * dh; ga[r][2] += gv * dw;
+                                } else {
+                                    const T fh = misc[0], gh = (T)1 - fh, fw = misc[1], gw = (T)1 - fw;
+                                    ga[r][0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
+                                    ga[r][1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
+                                }
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) atomic_add(gin_n + ix[i], sCw[wave][rho][i] * gv);
+                            } else if constexpr (ND == 3) {
+                                const T av = gv > 0 ? gv : -gv;
+#pragma unroll
+                                for (int a = 0; a < ND; ++a) ga[r][a] += misc[3 + a] * av;
                             }
-#pragma unroll
-                            for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
-                        } else if (ND == 3 && any_oob) {
-                            const T av = gv > 0 ? gv : -gv;
-#pragma unroll
-                            for (int a = 0; a < ND; ++a) ga[a] += oob[a] * av;
                         }
                     }
                 }
             }
         }
-        // sum the partial results of the KL lane groups that share a position, then one
-        // coalesced store per axis
+        // per position: sum over the channel lanes, then the lanes that hold the sums store
+        // them, lane <-> register r, i.e. position row(r, q)
 #pragma unroll
         for (int a = 0; a < ND; ++a) {
+            T mine = 0;
 #pragma unroll
-            for (int sh = TN; sh < 64; sh <<= 1) ga[a] += __shfl_xor(ga[a], sh);
-            if (q == 0 && valid) goff_dg[((size_t)tap * ND + a) * P.outV + pos] = ga[a];
+            for (int r = 0; r < NACC; ++r) {
+                const T s = group_sum(ga[r][a]);
+                if ((j % 16) == r) mine = s;
+            }
+            const int r_mine = j % 16;
+            if (sum_holder<T>(j) && r_mine < NACC && (TN == 32 || j < 16)) {
+                const unsigned p_out = pos0 + MM::row(r_mine, q);
+                if (p_out < P.outV) goff_dg[((size_t)tap * ND + a) * P.outV + p_out] = mine;
+            }
         }
     }
 }

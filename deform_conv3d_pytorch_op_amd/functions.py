@@ -90,7 +90,10 @@ def _workspace(inputs, weight, group):
     kV = 1
     for k in weight.shape[2:]:
         kV *= k
-    nbytes = L.dcn_workspace_bytes(inputs.element_size(), inputs.size(1), weight.size(0), kV, group)
+    inV = 1
+    for v in inputs.shape[2:]:
+        inV *= v
+    nbytes = L.dcn_workspace_bytes(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, kV, group)
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=inputs.device), int(nbytes)
 
 

@@ -26,8 +26,8 @@
  *
  * Differences from the reference ABI, all on purpose:
  *   - there is no `columns` argument: the sampled column buffer never exists in device memory;
- *   - `workspace` is caller-owned scratch of at least dcn_workspace_bytes(...) bytes (it holds a
- *     re-laid-out copy of the weights); the library never allocates device memory;
+ *   - `workspace` is caller-owned scratch of at least dcn_workspace_bytes(...) bytes, 256-byte
+ *     aligned; the library never allocates device memory;
  *   - `stream` is the hipStream_t to enqueue on (NULL = the null stream); calls are asynchronous;
  *   - the return value is 0 on success and a negative DCN_E_* code on failure, with the text
  *     from dcn_last_error() (thread-local).  The reference returns 1 and raises through THError.
@@ -58,8 +58,12 @@ int dcn_version(void);              /* ABI version, currently 1 */
 const char *dcn_arch(void);         /* the code-object target the kernels were built for: "gfx950" */
 const char *dcn_last_error(void);   /* message of the last failing call on this thread ("" if none) */
 
-/* Scratch bytes any of the three calls below needs for this layer (elem_size 4 = f32, 8 = f64). */
-size_t dcn_workspace_bytes(int elem_size, int input_c, int output_c, int kernel_volume, int group);
+/* Scratch bytes any of the three calls below needs for this layer (elem_size 4 = f32, 8 = f64;
+ * input_volume = input_l * input_h * input_w, kernel_volume = kernel_l * kernel_h * kernel_w).
+ * The workspace holds a re-laid-out copy of the weight and, for backward_input_offset,
+ * channels-last copies of one input batch and of its gradient. */
+size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
+                           int kernel_volume, int group);
 
 /* ---- 3-D, trilinear ------------------------------------------------------------------------
  * replaces deform3d/lib/deform_conv3d_cuda.cpp:90-165 (forward), :168-262 (backward_input_offset)
