@@ -5,6 +5,7 @@
 #include "dcn_kernels.h"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 
@@ -104,6 +105,67 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 }
 
 // ---------------------------------------------------------------------------------------------
+// Halo tiling plan: block of output positions per workgroup, halo extents, channels per LDS pass.
+// Returns false when the geometry does not suit (halo too large for the staging table or LDS).
+constexpr size_t LDS_BUDGET = 144 * 1024;       // of the 160 KB per CU
+int g_halo_margin = -1;                          // test hook: DCN_HALO_MARGIN overrides the default of 2
+
+int halo_margin() {
+    if (g_halo_margin < 0) {
+        const char* e = getenv("DCN_HALO_MARGIN");
+        g_halo_margin = e ? atoi(e) : 2;
+        if (g_halo_margin < 0) g_halo_margin = 0;
+    }
+    return g_halo_margin;
+}
+
+template <typename T, int ND>
+bool plan_halo(Params& P, size_t budget) {
+    const int npos = WAVESH * Mma<T>::TN;       // positions per workgroup: 256 (float) or 128 (double)
+    int td[3] = {1, 1, 1};
+    if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
+    else         { td[2] = 16; td[1] = npos / 16; }
+    const int m = halo_margin();
+    long long hvol = 1, tiles = 1;
+    for (int a = 0; a < 3; ++a) {
+        P.tdim[a] = td[a];
+        P.ntile[a] = (P.out[a] + td[a] - 1) / td[a];
+        const bool used = a >= 3 - ND;
+        P.mlo[a] = used ? m : 0;
+        // lowest corner: base - m; highest corner: base + m (the high corner of a sample at base + m - eps)
+        P.hext[a] = used ? (td[a] - 1) * P.stride[a] + (P.k[a] - 1) * P.dil[a] + 1 + 2 * m : 1;
+        hvol *= P.hext[a];
+        tiles *= P.ntile[a];
+    }
+    if (hvol > (long long)WGH * NSTG) return false;
+    P.hvol = (int)hvol;
+    P.hstride = ((int)hvol + 63) / 64 * 64 + 32;
+    const int KL = Mma<T>::KL;
+    long long cc = (long long)(budget / ((size_t)P.hstride * sizeof(T)));
+    cc = cc / KL * KL;
+    const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;          // longest run of channels sharing offsets and group
+    const int seg_up = (seg + KL - 1) / KL * KL;
+    if (cc > seg_up) cc = seg_up;
+    if (cc < KL) return false;
+    P.cchunk = (int)cc;
+    if (tiles * P.N > 0x7fffffffLL) return false;
+    P.tiles = (int)tiles;
+    return true;
+}
+
+template <typename K, typename... Args>
+int launch_halo(K kern, const char* name, dim3 grid, size_t lds, hipStream_t s, Args... args) {
+    if (lds > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
+        }
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(WGH), lds, s, args...);
+    return check_launch(name);
+}
+
 template <typename T, int ND>
 int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* bias, T* out, void* ws,
             size_t ws_bytes, hipStream_t s) {
@@ -116,6 +178,17 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     T* wt = static_cast<T*>(ws);
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     const int TN = Mma<T>::TN;
+    if (plan_halo<T, ND>(P, LDS_BUDGET)) {
+        const size_t lds = (size_t)P.cchunk * P.hstride * sizeof(T);
+        const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
+        switch (MT) {
+            case 1: return launch_halo(forward_halo_kernel<T, ND, 1>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
+            case 2: return launch_halo(forward_halo_kernel<T, ND, 2>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
+            case 4: return launch_halo(forward_halo_kernel<T, ND, 4>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
+            default: return launch_halo(forward_halo_kernel<T, ND, 8>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
+        }
+    }
+    // geometry whose halo does not fit in LDS: gather straight from global memory
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
     switch (MT) {

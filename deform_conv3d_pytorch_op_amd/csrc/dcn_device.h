@@ -23,6 +23,14 @@ struct Params {
     int Mp, Cgp;                  // padded extents of the re-laid-out weight in the workspace
     int nsplit;                   // backward-weight: number of position splits
     int nctiles;                  // backward-weight: channel tiles over all (group, deformable group) segments
+    // LDS halo tiling (kernels that stage an input neighbourhood in LDS); slots as in[] / out[]
+    int tdim[3];                  // output positions per workgroup tile along each axis
+    int ntile[3];                 // tiles along each axis
+    int hext[3];                  // halo extent in input voxels along each axis
+    int mlo[3];                   // halo margin below the lowest integer tap coordinate
+    int hvol;                     // hext[0] * hext[1] * hext[2]
+    int hstride;                  // LDS elements between the planes of two channels (>= hvol)
+    int cchunk;                   // channels staged per pass
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -97,6 +105,7 @@ struct TapGeo {
     unsigned idx[NC];   // voxel offset of each corner inside one channel; corner bit (ND-1-a) = high on axis a
     T f[ND];            // fraction toward the high corner on each axis
     T p[ND];            // absolute sampling coordinate
+    int lo[ND], hi[ND]; // low / high corner coordinate per axis
     bool inside;        // strict -1 < p < size on every axis
 };
 
@@ -122,6 +131,8 @@ __device__ inline void tap_setup(const Params& P, const T* __restrict__ off_tap,
         t.f[a] = p - (T)l;
     }
     t.inside = inside;
+#pragma unroll
+    for (int a = 0; a < ND; ++a) { t.lo[a] = lo[a]; t.hi[a] = hi[a]; }
     if constexpr (ND == 3) {
         const unsigned s1 = P.in[2], s2 = P.in[1] * P.in[2];
 #pragma unroll

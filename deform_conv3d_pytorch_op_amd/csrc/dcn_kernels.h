@@ -112,6 +112,213 @@ __global__ __launch_bounds__(WG) void forward_kernel(Params P, const T* __restri
 }
 
 // ---------------------------------------------------------------------------------------------
+// Halo tiling.  A workgroup of WGH threads owns a compact block of output positions
+// (tdim[0] x tdim[1] x tdim[2], WAVESH * TN of them) and stages the input neighbourhood that the
+// block's samples can reach -- the "halo" -- in LDS, `cchunk` channels at a time, as channel
+// planes [channel][halo voxel].  Samples whose corners all fall inside the halo are interpolated
+// from LDS; the few that reach further (large offsets) fall back to global memory, so any offset
+// field is handled and only the speed depends on it.
+constexpr int WGH = 512;
+constexpr int WAVESH = WGH / 64;
+constexpr int NSTG = 6;            // halo voxels staged per thread and channel: hvol <= WGH * NSTG
+
+template <int ND>
+struct TileGeo {
+    int n;              // sample
+    int o0[ND];         // first output position of the tile
+    int hb[ND];         // input coordinate of halo voxel (0,0,0)
+};
+
+template <int ND>
+__device__ inline void tile_decode(const Params& P, unsigned bid, TileGeo<ND>& tg) {
+    unsigned t = bid % (unsigned)P.tiles;
+    tg.n = bid / (unsigned)P.tiles;
+#pragma unroll
+    for (int a = ND - 1; a >= 0; --a) {
+        const int s = slot<ND>(a);
+        const int ti = t % P.ntile[s];
+        t /= P.ntile[s];
+        tg.o0[a] = ti * P.tdim[s];
+        tg.hb[a] = tg.o0[a] * P.stride[s] - P.pad[s] - P.mlo[s];
+    }
+}
+
+// position `pt` (0 .. tile volume - 1) of the tile -> output coordinate; returns validity and the
+// linear position (clamped into the volume so that offset loads of masked lanes stay legal)
+template <int ND>
+__device__ inline bool tile_position(const Params& P, const TileGeo<ND>& tg, int pt, int o[ND], unsigned& pos) {
+    bool valid = true;
+#pragma unroll
+    for (int a = ND - 1; a >= 0; --a) {
+        const int s = slot<ND>(a);
+        const int loc = pt % P.tdim[s];
+        pt /= P.tdim[s];
+        int oa = tg.o0[a] + loc;
+        if (oa >= P.out[s]) { valid = false; oa = P.out[s] - 1; }
+        o[a] = oa;
+    }
+    unsigned lin = 0;
+#pragma unroll
+    for (int a = 0; a < ND; ++a) lin = lin * (unsigned)P.out[slot<ND>(a)] + (unsigned)o[a];
+    pos = lin;
+    return valid;
+}
+
+// voxel offsets (inside one channel) of the halo elements this thread stages, ~0u where the
+// halo sticks out of the volume
+template <int ND>
+__device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsigned goff[NSTG]) {
+#pragma unroll
+    for (int k = 0; k < NSTG; ++k) {
+        int v = threadIdx.x + WGH * k;
+        unsigned g = ~0u;
+        if (v < P.hvol) {
+            bool inb = true;
+            unsigned lin = 0;
+            int c[ND];
+#pragma unroll
+            for (int a = ND - 1; a >= 0; --a) {
+                const int s = slot<ND>(a);
+                c[a] = tg.hb[a] + v % P.hext[s];
+                v /= P.hext[s];
+                inb = inb && c[a] >= 0 && c[a] < P.in[s];
+            }
+#pragma unroll
+            for (int a = 0; a < ND; ++a) lin = lin * (unsigned)P.in[slot<ND>(a)] + (unsigned)c[a];
+            if (inb) g = lin;
+        }
+        goff[k] = g;
+    }
+}
+
+template <typename T>
+__device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, int nch, const unsigned goff[NSTG],
+                                  T* __restrict__ sIn) {
+    for (int c = 0; c < nch; ++c) {
+        const T* ch = chan0 + (size_t)c * P.inV;
+#pragma unroll
+        for (int k = 0; k < NSTG; ++k)
+            if (goff[k] != ~0u) sIn[c * P.hstride + threadIdx.x + WGH * k] = ch[goff[k]];
+    }
+}
+
+// LDS indices of the corners of an inside sample; false if any corner lies outside the halo
+template <typename T, int ND>
+__device__ inline bool halo_corners(const Params& P, const int hb[ND], const TapGeo<T, ND>& t, unsigned lidx[1 << ND]) {
+    bool in_halo = true;
+    int l[ND], h[ND];
+#pragma unroll
+    for (int a = 0; a < ND; ++a) {
+        l[a] = t.lo[a] - hb[a];
+        h[a] = t.hi[a] - hb[a];
+        in_halo = in_halo && l[a] >= 0 && h[a] < P.hext[slot<ND>(a)];
+    }
+    if constexpr (ND == 3) {
+        const int e1 = P.hext[1], e2 = P.hext[2];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            lidx[c] = in_halo ? (unsigned)((((c & 4) ? h[0] : l[0]) * e1 + ((c & 2) ? h[1] : l[1])) * e2 + ((c & 1) ? h[2] : l[2])) : 0u;
+    } else {
+        const int e2 = P.hext[2];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            lidx[c] = in_halo ? (unsigned)(((c & 2) ? h[0] : l[0]) * e2 + ((c & 1) ? h[1] : l[1])) : 0u;
+    }
+    return in_halo;
+}
+
+// Forward with the input halo in LDS.  Same contraction and lane roles as forward_kernel; the
+// sampled value of lane (j, q) is the MFMA B operand B[k = q][col = j].
+// grid.x = N * tiles (3-D blocks of positions), grid.y = G * mchunks; dynamic LDS = cchunk * hstride * sizeof(T).
+template <typename T, int ND, int MT>
+__global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __restrict__ in,
+                                                           const T* __restrict__ off, const T* __restrict__ Wt,
+                                                           const T* __restrict__ bias, T* __restrict__ out) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sIn = reinterpret_cast<T*>(smem_raw);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % TN, q = lane / TN;
+    const int g = blockIdx.y / P.mchunks, mchunk = blockIdx.y % P.mchunks;
+
+    TileGeo<ND> tg;
+    tile_decode<ND>(P, blockIdx.x, tg);
+    const int n = tg.n;
+    int o[ND], ib[ND];
+    unsigned pos;
+    const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
+#pragma unroll
+    for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
+    unsigned goff[NSTG];
+    halo_table<ND>(P, tg, goff);
+
+    typename MM::Acc acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
+
+    const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
+    for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+        const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
+        const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+        for (int cc0 = cb; cc0 < ce; cc0 += P.cchunk) {
+            const int nch = min(P.cchunk, ce - cc0);
+            const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
+            __syncthreads();                                               // readers of the previous chunk are done
+            halo_stage<T>(P, chan0, nch, goff, sIn);
+            __syncthreads();
+            const int nsteps = (nch + KL - 1) / KL;
+            for (int tap = 0; tap < P.kV; ++tap) {
+                int kk[ND], kd[ND];
+                decode_tap<ND>(P, tap, kk);
+#pragma unroll
+                for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+                TapGeo<T, ND> t;
+                tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, pos, ib, kd, t);
+                const bool live = valid && t.inside;
+                if (!__any(live)) continue;        // whole wave outside: these column rows are zero
+                unsigned lidx[NC], voff[NC];
+                const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    lidx[c] += (unsigned)q * P.hstride;
+                    voff[c] = t.idx[c] + (unsigned)q * P.inV;
+                }
+                const T* plane = sIn;
+                const T* chan = chan0;
+                const T* wrow = Wt + (((size_t)g * P.kV + tap) * P.Cgp + (cc0 - cg0) + q) * P.Mp +
+                                (size_t)mchunk * MT * TN + j;
+                for (int s = 0; s < nsteps; ++s) {
+                    T b = 0;
+                    if (live && s * KL + q < nch) {
+                        if (in_halo) b = sample<T, ND>(plane, lidx, t.f);
+                        else b = sample<T, ND>(chan, voff, t.f);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wrow[mt * TN], b, acc[mt]);
+                    plane += KL * P.hstride;
+                    chan += (size_t)KL * P.inV;
+                    wrow += (size_t)KL * P.Mp;
+                }
+            }
+        }
+    }
+
+    if (!valid) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < MM::NACC; ++r) {
+            const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
+            if (m < P.M) {
+                T v = acc[mt][r];
+                if (bias) v += bias[g * P.M + m];
+                out[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Layout changes between [C][V] (channel planes, what PyTorch hands over) and [V][C]
 // (channels-last, what the scatter / coordinate kernel wants so that the lanes of a wavefront
 // touch consecutive addresses).  32x32 tiles through LDS; grid (ceil(V/32), ceil(C/32), N),
