@@ -28,7 +28,7 @@ template <typename T> void fwd_weight_pad(int M, int Cg, int& MT, int& mchunks, 
     MT = mtiles >= 8 ? 8 : (mtiles > 2 ? 4 : mtiles);          // 1, 2, 4 or 8 tiles per wavefront
     mchunks = (mtiles + MT - 1) / MT;
     Mp = mchunks * MT * TN;
-    Cgp = Cg + KL;
+    Cgp = Cg + 2 * KL;       // the kernels read up to one reduction step past the last channel
 }
 template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp) {
     Mp = M + Mma<T>::KL;

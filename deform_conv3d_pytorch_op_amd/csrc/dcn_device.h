@@ -109,12 +109,32 @@ struct TapGeo {
     bool inside;        // strict -1 < p < size on every axis
 };
 
-// `off_tap` points at offset[n][dg][tap][0][0]; `ib[a]` is out*stride - pad of this lane's
-// position, `kd[a]` is tap*dilation (wave-uniform).  Corner indices are only meaningful when
-// `inside`; otherwise they are zero so that a masked-off lane never forms a wild address.
+// `offv[a]` is the learned offset of this (tap, position) on axis a, `ib[a]` is out*stride - pad
+// of this lane's position, `kd[a]` is tap*dilation (wave-uniform).  Corner indices are only
+// meaningful when `inside`; otherwise they are zero so that a masked-off lane never forms a wild
+// address.
+template <typename T, int ND>
+__device__ inline void load_offsets(const Params& P, const T* __restrict__ off_tap, unsigned pos, T offv[ND]) {
+#pragma unroll
+    for (int a = 0; a < ND; ++a) offv[a] = off_tap[(size_t)a * P.outV + pos];
+}
+
+template <typename T, int ND>
+__device__ inline void tap_setup(const Params& P, const T offv[ND], const int ib[ND], const int kd[ND],
+                                 TapGeo<T, ND>& t);
+
+// convenience form: `off_tap` points at offset[n][dg][tap][0][0]
 template <typename T, int ND>
 __device__ inline void tap_setup(const Params& P, const T* __restrict__ off_tap, unsigned pos,
                                  const int ib[ND], const int kd[ND], TapGeo<T, ND>& t) {
+    T offv[ND];
+    load_offsets<T, ND>(P, off_tap, pos, offv);
+    tap_setup<T, ND>(P, offv, ib, kd, t);
+}
+
+template <typename T, int ND>
+__device__ inline void tap_setup(const Params& P, const T offv[ND], const int ib[ND], const int kd[ND],
+                                 TapGeo<T, ND>& t) {
     bool inside = true;
     int lo[ND], hi[ND];
 #pragma unroll
@@ -122,7 +142,7 @@ __device__ inline void tap_setup(const Params& P, const T* __restrict__ off_tap,
         const int size = P.in[slot<ND>(a)];
         // integer part formed in int and converted once, then the offset is added (reference:
         // `l_in + l_kernel*dilation_l + data_offset_base_ptr[...]`)
-        const T p = (T)(ib[a] + kd[a]) + off_tap[(size_t)a * P.outV + pos];
+        const T p = (T)(ib[a] + kd[a]) + offv[a];
         t.p[a] = p;
         inside = inside && (p > (T)-1) && (p < (T)size);
         const int l = (int)p;                                   // truncation toward zero

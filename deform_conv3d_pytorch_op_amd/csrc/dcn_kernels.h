@@ -164,8 +164,9 @@ __device__ inline bool tile_position(const Params& P, const TileGeo<ND>& tg, int
     return valid;
 }
 
-// voxel offsets (inside one channel) of the halo elements this thread stages, ~0u where the
-// halo sticks out of the volume
+// voxel offsets (inside one channel) of the halo elements this thread stages.  Halo voxels that
+// stick out of the volume are never read by a sample, so they are simply staged from voxel 0
+// (keeps every load unconditional); slots past the halo volume are marked ~0u and skipped.
 template <int ND>
 __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsigned goff[NSTG]) {
 #pragma unroll
@@ -185,7 +186,7 @@ __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsign
             }
 #pragma unroll
             for (int a = 0; a < ND; ++a) lin = lin * (unsigned)P.in[slot<ND>(a)] + (unsigned)c[a];
-            if (inb) g = lin;
+            g = inb ? lin : 0u;
         }
         goff[k] = g;
     }
@@ -196,9 +197,12 @@ __device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, 
                                   T* __restrict__ sIn) {
     for (int c = 0; c < nch; ++c) {
         const T* ch = chan0 + (size_t)c * P.inV;
+        T v[NSTG];
+#pragma unroll
+        for (int k = 0; k < NSTG; ++k) v[k] = ch[goff[k] == ~0u ? 0u : goff[k]];     // all loads in flight together
 #pragma unroll
         for (int k = 0; k < NSTG; ++k)
-            if (goff[k] != ~0u) sIn[c * P.hstride + threadIdx.x + WGH * k] = ch[goff[k]];
+            if (goff[k] != ~0u) sIn[c * P.hstride + threadIdx.x + WGH * k] = v[k];
     }
 }
 
@@ -268,37 +272,67 @@ __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __
             halo_stage<T>(P, chan0, nch, goff, sIn);
             __syncthreads();
             const int nsteps = (nch + KL - 1) / KL;
+            T onext[ND];
+            load_offsets<T, ND>(P, off_dg, pos, onext);                    // offsets of tap 0
             for (int tap = 0; tap < P.kV; ++tap) {
                 int kk[ND], kd[ND];
                 decode_tap<ND>(P, tap, kk);
 #pragma unroll
                 for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+                T ocur[ND];
+#pragma unroll
+                for (int a = 0; a < ND; ++a) ocur[a] = onext[a];
+                // the next tap's offsets travel while this tap is computed
+                if (tap + 1 < P.kV) load_offsets<T, ND>(P, off_dg + (size_t)(tap + 1) * ND * P.outV, pos, onext);
                 TapGeo<T, ND> t;
-                tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, pos, ib, kd, t);
+                tap_setup<T, ND>(P, ocur, ib, kd, t);
                 const bool live = valid && t.inside;
                 if (!__any(live)) continue;        // whole wave outside: these column rows are zero
-                unsigned lidx[NC], voff[NC];
+                unsigned lidx[NC];
                 const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+                const bool near = live && in_halo;                         // sampled from LDS
+                const bool far = live && !in_halo;                         // sampled from global memory
 #pragma unroll
-                for (int c = 0; c < NC; ++c) {
-                    lidx[c] += (unsigned)q * P.hstride;
-                    voff[c] = t.idx[c] + (unsigned)q * P.inV;
-                }
-                const T* plane = sIn;
-                const T* chan = chan0;
+                for (int c = 0; c < NC; ++c) lidx[c] += (unsigned)q * P.hstride;   // 0 + plane of this lane when !in_halo
                 const T* wrow = Wt + (((size_t)g * P.kV + tap) * P.Cgp + (cc0 - cg0) + q) * P.Mp +
                                 (size_t)mchunk * MT * TN + j;
-                for (int s = 0; s < nsteps; ++s) {
-                    T b = 0;
-                    if (live && s * KL + q < nch) {
-                        if (in_halo) b = sample<T, ND>(plane, lidx, t.f);
-                        else b = sample<T, ND>(chan, voff, t.f);
-                    }
+                // branch-free main loop: every lane reads LDS at a legal index and the value is
+                // masked afterwards; the weights of the next step are fetched one step ahead
+                {
+                    const T* plane = sIn;
+                    const T* wr = wrow;
+                    T a_next[MT];
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wrow[mt * TN], b, acc[mt]);
-                    plane += KL * P.hstride;
-                    chan += (size_t)KL * P.inV;
-                    wrow += (size_t)KL * P.Mp;
+                    for (int mt = 0; mt < MT; ++mt) a_next[mt] = wr[mt * TN];
+#pragma unroll 2
+                    for (int s = 0; s < nsteps; ++s) {
+                        T a_cur[MT];
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) a_cur[mt] = a_next[mt];
+                        wr += (size_t)KL * P.Mp;                           // rows past the chunk stay inside the padded weight
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) a_next[mt] = wr[mt * TN];
+                        const T v = sample<T, ND>(plane, lidx, t.f);
+                        const T b = (near && s * KL + q < nch) ? v : (T)0;
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a_cur[mt], b, acc[mt]);
+                        plane += KL * P.hstride;
+                    }
+                }
+                if (__any(far)) {                  // rare: some sample of this wave reaches past the halo
+                    unsigned voff[NC];
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
+                    const T* chan = chan0;
+                    const T* wr = wrow;
+                    for (int s = 0; s < nsteps; ++s) {
+                        T b = 0;
+                        if (far && s * KL + q < nch) b = sample<T, ND>(chan, voff, t.f);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wr[mt * TN], b, acc[mt]);
+                        chan += (size_t)KL * P.inV;
+                        wr += (size_t)KL * P.Mp;
+                    }
                 }
             }
         }
