@@ -125,7 +125,7 @@ def main():
     suf = "f32" if dtype == torch.float32 else "f64"
     geom = _geom(nd, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
     nbytes = L.dcn_workspace_bytes(x.element_size(), x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]),
-                                   math.prod(c["k"]), c["groups"])
+                                   math.prod(c["outs"]), math.prod(c["k"]), c["groups"])
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     out = torch.empty((x.shape[0], w.shape[0]) + c["outs"], dtype=dtype, device=dev)
     gin, goff, gw = torch.zeros_like(x), torch.empty_like(off), torch.zeros_like(w)
@@ -139,7 +139,7 @@ def main():
             xd.data_ptr(), wd.data_ptr(), od.data_ptr(), gout.data_ptr(), gin.data_ptr(), goff.data_ptr(), *geom,
             ws.data_ptr(), nbytes, sp),
         "backward_weight": lambda: getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))(
-            xd.data_ptr(), od.data_ptr(), gout.data_ptr(), gw.data_ptr(), *geom, None, 0, sp),
+            xd.data_ptr(), od.data_ptr(), gout.data_ptr(), gw.data_ptr(), *geom, ws.data_ptr(), nbytes, sp),
     }
     kernel_ms = {}
     for name, call in calls.items():

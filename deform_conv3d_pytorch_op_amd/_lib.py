@@ -35,7 +35,7 @@ def load():
     L.dcn_arch.restype = ctypes.c_char_p
     L.dcn_last_error.restype = ctypes.c_char_p
     L.dcn_workspace_bytes.restype = _c_sz
-    L.dcn_workspace_bytes.argtypes = [_c_int] * 4 + [_c_sz, _c_int, _c_int]
+    L.dcn_workspace_bytes.argtypes = [_c_int] * 4 + [_c_sz, _c_sz, _c_int, _c_int]
     tail = [_c_vp, _c_sz, _c_vp]            # workspace, workspace_bytes, stream
     for nd in (2, 3):
         geom = [_c_int] * N_GEOM[nd]

@@ -30,8 +30,18 @@ template <typename T> void fwd_weight_pad(int M, int Cg, int& MT, int& mchunks, 
     Mp = mchunks * MT * TN;
     Cgp = Cg + 2 * KL;       // the kernels read up to one reduction step past the last channel
 }
+// backward-data layout.  MK = reduction steps over output channels kept in registers by
+// backward_input_halo_kernel (0: M too large, the kernel re-reads grad_output per tap).
+template <typename T> int bwd_data_mk(int M) {
+    const int steps = (M + Mma<T>::KL - 1) / Mma<T>::KL;
+    for (int mk = 8; mk <= 64; mk *= 2)
+        if (steps <= mk) return mk;
+    return 0;
+}
 template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp) {
+    const int mk = bwd_data_mk<T>(M) * Mma<T>::KL;
     Mp = M + Mma<T>::KL;
+    if (mk > Mp) Mp = mk;
     Cgp = Cg + Mma<T>::TN;
 }
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
@@ -42,13 +52,15 @@ template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G)
     bwd_data_weight_pad<T>(M, Cg, Mp, Cgp);
     return align256((size_t)G * kV * Mp * Cgp * sizeof(T));
 }
-template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, int kV, int G) {
+template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G) {
     const int M = C_out / G, Cg = C_in / G;
     int MT, mchunks, Mp, Cgp;
     fwd_weight_pad<T>(M, Cg, MT, mchunks, Mp, Cgp);
     const size_t fwd = (size_t)G * kV * Mp * Cgp * sizeof(T);
     const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
-    return fwd > bwd ? fwd : bwd;
+    const size_t bww = align256((size_t)N * C_in * inV * sizeof(T)) + align256((size_t)N * C_out * outV * sizeof(T));
+    size_t need = fwd > bwd ? fwd : bwd;
+    return need > bww ? need : bww;
 }
 
 struct Geometry {   // the reference's argument list, 2-D mapped onto slots 1,2 with a unit length axis
@@ -107,7 +119,8 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 // ---------------------------------------------------------------------------------------------
 // Halo tiling plan: block of output positions per workgroup, halo extents, channels per LDS pass.
 // Returns false when the geometry does not suit (halo too large for the staging table or LDS).
-constexpr size_t LDS_BUDGET = 144 * 1024;       // of the 160 KB per CU
+static size_t lds_budget() { const char* e = getenv("DCN_LDS_BUDGET_KB"); return (size_t)(e ? atoi(e) : 72) * 1024; }
+#define LDS_BUDGET lds_budget()
 int g_halo_margin = -1;                          // test hook: DCN_HALO_MARGIN overrides the default of 2
 
 int halo_margin() {
@@ -120,7 +133,7 @@ int halo_margin() {
 }
 
 template <typename T, int ND>
-bool plan_halo(Params& P, size_t budget) {
+bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30) {
     const int npos = WAVESH * Mma<T>::TN;       // positions per workgroup: 256 (float) or 128 (double)
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
@@ -146,6 +159,7 @@ bool plan_halo(Params& P, size_t budget) {
     const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;          // longest run of channels sharing offsets and group
     const int seg_up = (seg + KL - 1) / KL * KL;
     if (cc > seg_up) cc = seg_up;
+    if (cc > max_chunk) cc = max_chunk / KL * KL;
     if (cc < KL) return false;
     P.cchunk = (int)cc;
     if (tiles * P.N > 0x7fffffffLL) return false;
@@ -217,41 +231,76 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     const dim3 tgrid((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N), tblock(32, 8);
     hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
+    const int TN = Mma<T>::TN;
+    Params Ph = P;
+    const bool halo = plan_halo<T, ND>(Ph, LDS_BUDGET, TN) && getenv("DCN_LDS_SCATTER") != nullptr;
+    P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
+    const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
+    if (halo) {
+        // grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
+        T* none = nullptr;
+        switch (bwd_data_mk<T>(P.M)) {
+            case 8: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 8>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
+            case 16: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 16>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
+            case 32: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 32>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
+            case 64: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 64>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
+            default: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
+        }
+        if (int rc = check_launch("backward_data_kernel")) return rc;
+        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * sizeof(T);
+        const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
+        switch (bwd_data_mk<T>(P.M)) {
+            case 8: return launch_halo(backward_input_halo_kernel<T, ND, 8>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
+            case 16: return launch_halo(backward_input_halo_kernel<T, ND, 16>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
+            case 32: return launch_halo(backward_input_halo_kernel<T, ND, 32>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
+            case 64: return launch_halo(backward_input_halo_kernel<T, ND, 64>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
+            default: return launch_halo(backward_input_halo_kernel<T, ND, 0>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
+        }
+    }
+    // halo does not fit in LDS: scatter with global atomics on the channels-last copy
     const size_t nelem = (size_t)P.N * P.C_in * P.inV;
     const unsigned fblocks = (unsigned)((nelem + 1023) / 1024 > 8192 ? 8192 : (nelem + 1023) / 1024);
     hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fblocks), dim3(256), 0, s, gin_cl, nelem);
     if (int rc = check_launch("fill_zero_kernel")) return rc;
-    const int TN = Mma<T>::TN;
-    P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
-    const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
-    hipLaunchKernelGGL((backward_data_kernel<T, ND>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff);
+    switch (bwd_data_mk<T>(P.M)) {
+        case 8: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 8>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
+        case 16: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 16>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
+        case 32: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 32>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
+        case 64: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 64>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
+        default: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
+    }
     if (int rc = check_launch("backward_data_kernel")) return rc;
     hipLaunchKernelGGL(add_from_channels_last_kernel<T>, tgrid, tblock, 0, s, gin_cl, gin, P.C_in, P.inV);
     return check_launch("add_from_channels_last_kernel");
 }
 
 template <typename T, int ND, int MT>
-int launch_bwd_weight(const Params& P, const T* in, const T* off, const T* gout, T* gw, hipStream_t s) {
-    const int TN = Mma<T>::TN;
-    const size_t lds = (size_t)WAVES * (MT * TN + TN) * (TN + 1) * sizeof(T);
-    auto kern = backward_weight_kernel<T, ND, MT>;
-    if (lds > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit for backward_weight_kernel");
-        }
-    }
+int launch_bwd_weight(const Params& P, const T* in_cl, const T* off, const T* gout_cl, T* gw, hipStream_t s) {
     const dim3 grid((unsigned)P.nsplit, (unsigned)P.kV, (unsigned)(P.nctiles * P.mchunks));
-    hipLaunchKernelGGL(kern, grid, dim3(WG), lds, s, P, in, off, gout, gw);
+    hipLaunchKernelGGL((backward_weight_kernel<T, ND, MT>), grid, dim3(WG), 0, s, P, in_cl, off, gout_cl, gw);
     return check_launch("backward_weight_kernel");
 }
 
+// Workspace of backward_weight: [ input channels-last | grad_output channels-last ]
 template <typename T, int ND>
-int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout, T* gw, hipStream_t s) {
+int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout, T* gw, void* ws, size_t ws_bytes,
+                    hipStream_t s) {
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    if ((long long)P.outV * P.C_out > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one output sample exceeds 2^31 elements");
+    const size_t ibytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
+    const size_t obytes = align256((size_t)P.N * P.C_out * P.outV * sizeof(T));
+    if (!ws || ws_bytes < ibytes + obytes) return fail(DCN_E_WORKSPACE, "workspace too small");
+    T* in_cl = static_cast<T*>(ws);
+    T* gout_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + ibytes);
+    const dim3 tblock(32, 8);
+    hipLaunchKernelGGL(to_channels_last_kernel<T>, dim3((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N),
+                       tblock, 0, s, in, in_cl, P.C_in, P.inV);
+    if (int rc = check_launch("to_channels_last_kernel")) return rc;
+    hipLaunchKernelGGL(to_channels_last_kernel<T>, dim3((P.outV + 31) / 32, (unsigned)(P.C_out + 31) / 32, (unsigned)P.N),
+                       tblock, 0, s, gout, gout_cl, P.C_out, P.outV);
+    if (int rc = check_launch("to_channels_last_kernel")) return rc;
     const int TN = Mma<T>::TN;
     const int mtiles = (P.M + TN - 1) / TN;
     const int MT = mtiles > 2 ? 4 : mtiles;
@@ -277,9 +326,9 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     if (split < 1) split = 1;
     P.nsplit = (int)split;
     switch (MT) {
-        case 1: return launch_bwd_weight<T, ND, 1>(P, in, off, gout, gw, s);
-        case 2: return launch_bwd_weight<T, ND, 2>(P, in, off, gout, gw, s);
-        default: return launch_bwd_weight<T, ND, 4>(P, in, off, gout, gw, s);
+        case 1: return launch_bwd_weight<T, ND, 1>(P, in_cl, off, gout_cl, gw, s);
+        case 2: return launch_bwd_weight<T, ND, 2>(P, in_cl, off, gout_cl, gw, s);
+        default: return launch_bwd_weight<T, ND, 4>(P, in_cl, off, gout_cl, gw, s);
     }
 }
 
@@ -314,10 +363,13 @@ const char* dcn_arch(void) { return "gfx950"; }
 const char* dcn_last_error(void) { return g_err.c_str(); }
 
 size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
-                           int kernel_volume, int group) {
-    if (group <= 0 || batch <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0 || input_volume == 0) return 0;
-    return elem_size == 8 ? workspace_need<double>(batch, input_c, output_c, input_volume, kernel_volume, group)
-                          : workspace_need<float>(batch, input_c, output_c, input_volume, kernel_volume, group);
+                           size_t output_volume, int kernel_volume, int group) {
+    if (group <= 0 || batch <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0 || input_volume == 0 ||
+        output_volume == 0)
+        return 0;
+    return elem_size == 8
+               ? workspace_need<double>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group)
+               : workspace_need<float>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group);
 }
 
 #define DEFINE_OPS(SUF, T)                                                                                          \
@@ -335,9 +387,8 @@ size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, 
     }                                                                                                               \
     int dcn3d_backward_weight_##SUF(const T* input, const T* offset, const T* grad_output, T* grad_weight,          \
                                     DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {        \
-        (void)workspace; (void)workspace_bytes;                                                                     \
-        return backward_weight<T, 3>(geo3(G3_ARGS), input, offset, grad_output, grad_weight,                        \
-                                     static_cast<hipStream_t>(stream));                                             \
+        return backward_weight<T, 3>(geo3(G3_ARGS), input, offset, grad_output, grad_weight, workspace,             \
+                                     workspace_bytes, static_cast<hipStream_t>(stream));                            \
     }                                                                                                               \
     int dcn2d_forward_##SUF(const T* input, const T* weight, const T* offset, const T* bias, T* output,             \
                             DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {                \
@@ -353,9 +404,8 @@ size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, 
     }                                                                                                               \
     int dcn2d_backward_weight_##SUF(const T* input, const T* offset, const T* grad_output, T* grad_weight,          \
                                     DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {        \
-        (void)workspace; (void)workspace_bytes;                                                                     \
-        return backward_weight<T, 2>(geo2(G2_ARGS), input, offset, grad_output, grad_weight,                        \
-                                     static_cast<hipStream_t>(stream));                                             \
+        return backward_weight<T, 2>(geo2(G2_ARGS), input, offset, grad_output, grad_weight, workspace,             \
+                                     workspace_bytes, static_cast<hipStream_t>(stream));                            \
     }
 
 DEFINE_OPS(f32, float)

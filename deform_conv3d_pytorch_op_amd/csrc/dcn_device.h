@@ -193,5 +193,9 @@ __device__ inline T sample(const T* __restrict__ chan, const unsigned* voff, con
 
 __device__ inline void atomic_add(float* p, float v) { unsafeAtomicAdd(p, v); }
 __device__ inline void atomic_add(double* p, double v) { unsafeAtomicAdd(p, v); }
+// LDS float add without return value (ds_add_f32 / ds_add_f64)
+template <typename T> __device__ inline void lds_atomic_add(T* p, T v) {
+    (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
 
 }  // namespace dcn

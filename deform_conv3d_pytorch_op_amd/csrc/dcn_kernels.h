@@ -445,7 +445,10 @@ template <> __device__ inline bool sum_holder<double>(int) { return true; }
 // The geometry of a (tap, position) is computed once by the lane that owns the position and
 // handed to the channel lanes through LDS.
 // grid.x = N * tiles, grid.y = DG.  grad_offset gets a plain store of every element.
-template <typename T, int ND>
+// SCATTER = false leaves grad-input to backward_input_halo_kernel and only writes grad_offset.
+// MK > 0: the wavefront's grad_output slab (MK reduction steps of KL output channels) stays in
+// registers and the weight operands of a tile are fetched in one batch; MK == 0: any M.
+template <typename T, int ND, bool SCATTER, int MK>
 __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __restrict__ in_cl,
                                                            const T* __restrict__ off, const T* __restrict__ Wt,
                                                            const T* __restrict__ gout, T* __restrict__ gin_cl,
@@ -475,13 +478,30 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
     const T* in_n = in_cl + (size_t)n * P.inV * P.C_in;
     T* gin_n = gin_cl + (size_t)n * P.inV * P.C_in;
 
+    // grad_output slab of this wavefront: A[row = position j][k = output channel]
+    const int g_first = c_lo / P.Cg, g_last = (c_hi - 1) / P.Cg;
+    T greg[MK > 0 ? MK : 1];
+    auto load_slab = [&](int g) {
+        const T* gq = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + posc;
+#pragma unroll
+        for (int k = 0; k < (MK > 0 ? MK : 1); ++k)
+            greg[k] = (valid && k * KL + q < P.M) ? gq[(size_t)k * KL * P.outV] : (T)0;
+    };
+    if constexpr (MK > 0) load_slab(g_first);
+
+    T onext[ND];
+    load_offsets<T, ND>(P, off_dg, posc, onext);
     for (int tap = 0; tap < P.kV; ++tap) {
         int kk[ND], kd[ND];
         decode_tap<ND>(P, tap, kk);
 #pragma unroll
         for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+        T ocur[ND];
+#pragma unroll
+        for (int a = 0; a < ND; ++a) ocur[a] = onext[a];
+        if (tap + 1 < P.kV) load_offsets<T, ND>(P, off_dg + (size_t)(tap + 1) * ND * P.outV, posc, onext);
         TapGeo<T, ND> t;
-        tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, posc, ib, kd, t);
+        tap_setup<T, ND>(P, ocur, ib, kd, t);
         const bool live = valid && t.inside;
         T oob[3] = {0, 0, 0};
         if (ND == 3 && valid && !t.inside) {
@@ -523,19 +543,31 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
             for (int a = 0; a < ND; ++a) ga[r][a] = 0;
 
         if (work) {
-            for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
+            for (int g = g_first; g <= g_last; ++g) {
                 const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
                 const T* gb = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV + posc;
+                if constexpr (MK > 0) {
+                    if (g_first != g_last) load_slab(g);      // several convolution groups share this deformable group
+                }
                 for (int c0 = rb; c0 < re; c0 += TN) {
                     typename MM::Acc d = acc_zero<T>();
                     const T* wb = Wt + (((size_t)g * P.kV + tap) * P.Mp + q) * P.Cgp + (c0 - g * P.Cg) + j;
-                    const T* gq = gb + (size_t)q * P.outV;
-                    for (int m0 = 0; m0 < P.M; m0 += KL) {
-                        const T a = (valid && m0 + q < P.M) ? *gq : (T)0;      // A[row = position j][k = m]
-                        const T b = *wb;                                       // B[k = m][col = channel j]
-                        d = MM::mma(a, b, d);
-                        wb += (size_t)KL * P.Cgp;
-                        gq += (size_t)KL * P.outV;
+                    if constexpr (MK > 0) {
+                        T wreg[MK];                                            // B[k = m][col = channel j]
+#pragma unroll
+                        for (int k = 0; k < MK; ++k) wreg[k] = wb[(size_t)k * KL * P.Cgp];
+                        __builtin_amdgcn_sched_barrier(0);      // keep the loads batched ahead of the MFMA chain
+#pragma unroll
+                        for (int k = 0; k < MK; ++k) d = MM::mma(greg[k], wreg[k], d);
+                    } else {
+                        const T* gq = gb + (size_t)q * P.outV;
+                        for (int m0 = 0; m0 < P.M; m0 += KL) {
+                            const T a = (valid && m0 + q < P.M) ? *gq : (T)0;  // A[row = position j][k = m]
+                            const T b = *wb;                                   // B[k = m][col = channel j]
+                            d = MM::mma(a, b, d);
+                            wb += (size_t)KL * P.Cgp;
+                            gq += (size_t)KL * P.outV;
+                        }
                     }
                     const int c = c0 + j;
                     if (c < re) {
@@ -566,8 +598,10 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
                                     ga[r][0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
                                     ga[r][1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
                                 }
+                                if constexpr (SCATTER) {
 #pragma unroll
-                                for (int i = 0; i < NC; ++i) atomic_add(gin_n + ix[i], sCw[wave][rho][i] * gv);
+                                    for (int i = 0; i < NC; ++i) atomic_add(gin_n + ix[i], sCw[wave][rho][i] * gv);
+                                }
                             } else if constexpr (ND == 3) {
                                 const T av = gv > 0 ? gv : -gv;
 #pragma unroll
@@ -598,27 +632,168 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
 }
 
 // ---------------------------------------------------------------------------------------------
-// Backward to weight: gW[g*M+m][cl][tap] += sum_{n,pos} gout[n][g*M+m][pos] * sample(in[n][g*Cg+cl], tap, pos)
-// replaces the second deformable_im2col + Sgemm(beta=1) of deform3d/lib/deform_conv3d_cuda.cpp:283-320.
-// The reduction runs over positions, so both MFMA operands need lanes along the non-reduced
-// dimension (m, channel) while memory and the sampler are contiguous along positions: each
-// wavefront transposes its TN-position slab of grad_output and of sampled values through a
-// private LDS region.  A workgroup keeps one (tap, channel tile, m chunk) for its whole life and
-// strides over position slabs, so the [MT*TN x TN] accumulator stays in registers; partial sums
-// of different workgroups meet in grad_weight through hardware float atomics.
-// grid.x = nsplit, grid.y = kV, grid.z = nctiles * mchunks.
-template <typename T, int ND, int MT>
-__global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* __restrict__ in,
-                                                             const T* __restrict__ off,
-                                                             const T* __restrict__ gout, T* __restrict__ gw) {
+// Backward to input with the scatter privatised in LDS (col2im_input of the reference,
+// deform3d kernel.cu:229-296 / deform2d_double kernel.cu:201-238, fed by the grad-column GEMM of
+// deform3d/lib/deform_conv3d_cuda.cpp:213-220).
+//
+// Same halo tiling as forward_halo_kernel, but the LDS planes hold the partial grad-input of
+// `cchunk` (<= TN) channels over the halo of the workgroup's position block.  Per tap the
+// grad-column tile gcol[c][pos] (rows = the chunk's channels, lanes = positions) comes out of
+// MFMA; each lane adds its values to the 8 (4) corners with LDS float atomics
+// ((w_l*w_h*w_w)*gcol as in the reference).  After the 27 taps the planes are added to
+// grad_input with one hardware atomic per touched halo voxel -- about 1/30 of the global
+// atomics of a direct scatter.  Samples that reach past the halo use global atomics directly.
+// MK > 0: the wavefront's grad_output slab (MK reduction steps = M rounded up / KL) stays in
+// registers for the whole tile; MK == 0: it is re-read per tap (any M).
+// grid.x = N * tiles, grid.y = DG; dynamic LDS = cchunk * hstride * sizeof(T).
+template <typename T, int ND, int MK>
+__global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ off,
+                                                                  const T* __restrict__ Wt,
+                                                                  const T* __restrict__ gout,
+                                                                  T* __restrict__ gin) {
     using MM = Mma<T>;
-    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
-    constexpr int LD = TN + 1;                     // padded row: conflict-free transposed reads
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sG = reinterpret_cast<T*>(smem_raw);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
-    T* sA = reinterpret_cast<T*>(smem_raw) + (size_t)wave * (MT * TN + TN) * LD;   // [MT*TN][LD] grad_output slab
-    T* sB = sA + (size_t)MT * TN * LD;                                            // [TN][LD]    sampled slab
+    const int dg = blockIdx.y;
+
+    TileGeo<ND> tg;
+    tile_decode<ND>(P, blockIdx.x, tg);
+    const int n = tg.n;
+    int o[ND], ib[ND];
+    unsigned pos;
+    const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
+#pragma unroll
+    for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
+    unsigned goff[NSTG];
+    halo_table<ND>(P, tg, goff);
+
+    const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
+    const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+
+    for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
+        const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
+        const T* gq0 = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + pos;
+        T breg[MK > 0 ? MK : 1];
+        if constexpr (MK > 0) {
+#pragma unroll
+            for (int k = 0; k < MK; ++k)
+                breg[k] = (valid && k * KL + q < P.M) ? gq0[(size_t)k * KL * P.outV] : (T)0;
+        }
+        for (int cc0 = rb; cc0 < re; cc0 += P.cchunk) {
+            const int nch = min(P.cchunk, re - cc0);
+            __syncthreads();                        // the previous chunk's flush is done
+            for (int c = 0; c < nch; ++c)
+#pragma unroll
+                for (int k = 0; k < NSTG; ++k)
+                    if (goff[k] != ~0u) sG[c * P.hstride + threadIdx.x + WGH * k] = 0;
+            __syncthreads();
+
+            T onext[ND];
+            load_offsets<T, ND>(P, off_dg, pos, onext);
+            for (int tap = 0; tap < P.kV; ++tap) {
+                int kk[ND], kd[ND];
+                decode_tap<ND>(P, tap, kk);
+#pragma unroll
+                for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+                T ocur[ND];
+#pragma unroll
+                for (int a = 0; a < ND; ++a) ocur[a] = onext[a];
+                if (tap + 1 < P.kV) load_offsets<T, ND>(P, off_dg + (size_t)(tap + 1) * ND * P.outV, pos, onext);
+                TapGeo<T, ND> t;
+                tap_setup<T, ND>(P, ocur, ib, kd, t);
+                const bool live = valid && t.inside;
+                if (!__any(live)) continue;
+                unsigned lidx[NC];
+                const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+                const bool near = live && in_halo, far = live && !in_halo;
+                T cw[NC];
+                if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
+                    const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                    cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                    cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+                } else {
+                    const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                    cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                }
+                // grad-column tile: rows = channels cc0 + i, columns = this wavefront's positions
+                typename MM::Acc d = acc_zero<T>();
+                const T* wa = Wt + (((size_t)g * P.kV + tap) * P.Mp + q) * P.Cgp + (cc0 - g * P.Cg) + j;
+                if constexpr (MK > 0) {
+                    // all weight loads of the tile are issued before the first MFMA needs one
+                    T areg[MK];
+#pragma unroll
+                    for (int k = 0; k < MK; ++k) areg[k] = wa[(size_t)k * KL * P.Cgp];
+                    __builtin_amdgcn_sched_barrier(0);      // keep the loads batched ahead of the MFMA chain
+#pragma unroll
+                    for (int k = 0; k < MK; ++k) d = MM::mma(areg[k], breg[k], d);
+                } else {
+                    const T* gq = gq0;
+                    for (int m0 = 0; m0 < P.M; m0 += KL) {
+                        const T b = (valid && m0 + q < P.M) ? *gq : (T)0;
+                        d = MM::mma(*wa, b, d);
+                        wa += (size_t)KL * P.Cgp;
+                        gq += (size_t)KL * P.outV;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < NACC; ++r) {
+                    const int cl = MM::row(r, q);
+                    if (cl < nch) {
+                        const T gv = d[r];
+                        if (near) {
+                            T* plane = sG + cl * P.hstride;
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) lds_atomic_add(plane + lidx[i], cw[i] * gv);
+                        } else if (far) {
+                            T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
+                        }
+                    }
+                }
+            }
+            __syncthreads();                        // all LDS adds of this chunk have landed
+            for (int c = 0; c < nch; ++c) {
+                T* gc = gin + ((size_t)n * P.C_in + cc0 + c) * P.inV;
+#pragma unroll
+                for (int k = 0; k < NSTG; ++k)
+                    if (goff[k] != ~0u) {
+                        const T v = sG[c * P.hstride + threadIdx.x + WGH * k];
+                        if (v != (T)0) atomic_add(gc + goff[k], v);
+                    }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward to weight: gW[g*M+m][cl][tap] += sum_{n,pos} gout[n][g*M+m][pos] * sample(in[n][g*Cg+cl], tap, pos)
+// replaces the second deformable_im2col + Sgemm(beta=1) of deform3d/lib/deform_conv3d_cuda.cpp:283-320.
+// The reduction runs over positions, so both MFMA operands want lanes along the non-reduced
+// dimension: A[m][pos] and B[pos][channel].  With the input and grad_output held channels-last
+// ([voxel][channel], [position][out channel]) both operands are contiguous across the lanes of a
+// lane group: lane (j, q) samples channel c0 + j at position 2*ks + q of the slab (8 or 4
+// coalesced corner loads) and loads grad_output row m_base + j of the same position.  The
+// geometry of the slab's TN positions is computed once by the position-owning lanes and handed
+// to the channel lanes through a wavefront-private LDS record.
+// A workgroup keeps one (tap, channel tile, m chunk) for its whole life; its wavefronts stride
+// over position slabs independently (no workgroup barriers), so the [MT*TN x TN] accumulator
+// stays in registers; partial sums of different wavefronts meet in grad_weight through
+// hardware float atomics.
+// grid.x = nsplit, grid.y = kV, grid.z = nctiles * mchunks.
+template <typename T, int ND, int MT>
+__global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* __restrict__ in_cl,
+                                                             const T* __restrict__ off,
+                                                             const T* __restrict__ gout_cl, T* __restrict__ gw) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
+    __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // corner voxel index * C_in, 0 when the sample is dead
+    __shared__ __align__(16) T sF[WAVES][TN][4];             // f[ND]; [3] = 1 when the sample is live
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % TN, q = lane / TN;
 
     const int tap = blockIdx.y;
     const int mchunk = blockIdx.z % P.mchunks;
@@ -648,21 +823,26 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
 
+    const int m_base = mchunk * MT * TN;
+    const bool chan_ok = c0 + j < ce;
+    const unsigned cj = (unsigned)min(c0 + j, P.C_in - 1);          // clamped: dead lanes still load legally
+    unsigned mrow[MT];
+    bool m_ok[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m_base + mt * TN + j;
+        m_ok[mt] = m < P.M;
+        mrow[mt] = (unsigned)(g * P.M + min(m, P.M - 1));
+    }
+
     const int slabs_per_sample = (P.outV + TN - 1) / TN;
     const int nslabs = P.N * slabs_per_sample;
-    const int stride_slabs = gridDim.x * WAVES;
-    const int m_base = mchunk * MT * TN;
-    // uniform trip count for all wavefronts of the grid (the barriers below need it)
-    const int trips = (nslabs + stride_slabs - 1) / stride_slabs;
-    for (int it = 0; it < trips; ++it) {
-        const int slab = it * stride_slabs + blockIdx.x * WAVES + wave;
-        const bool slab_ok = slab < nslabs;
-        const int n = slab_ok ? slab / slabs_per_sample : 0;
-        const unsigned p0 = slab_ok ? (unsigned)(slab % slabs_per_sample) * TN : 0u;
+    for (int slab = blockIdx.x * WAVES + wave; slab < nslabs; slab += gridDim.x * WAVES) {
+        const int n = slab / slabs_per_sample;
+        const unsigned p0 = (unsigned)(slab % slabs_per_sample) * TN;
         const unsigned pos = p0 + j;
-        const bool valid = slab_ok && pos < P.outV;
+        const bool valid = pos < P.outV;
         const unsigned posc = valid ? pos : P.outV - 1;
-
         int o[ND], ib[ND];
         decode_pos<ND>(P, posc, o);
 #pragma unroll
@@ -671,33 +851,42 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
         tap_setup<T, ND>(P, off + (((size_t)n * P.DG + dg) * P.kV + tap) * ND * P.outV, posc, ib, kd, t);
         const bool live = valid && t.inside;
 
-        __syncthreads();        // previous slab's MFMA reads are done before LDS is overwritten
-        // grad_output slab: rows m_base .. m_base + MT*TN, lanes along positions (coalesced)
-        const T* gb = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV + posc;
-        for (int mr = q; mr < MT * TN; mr += KL) {
-            const int m = m_base + mr;
-            sA[mr * LD + j] = (valid && m < P.M) ? gb[(size_t)m * P.outV] : (T)0;
-        }
-        // sampled slab: channel c0 + cr for cr in [0, TN)
-        unsigned voff[NC];
+        // LDS operations of one wavefront execute in order; the fences only pin the compiler
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (q == 0) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
-        const T* chan = in + ((size_t)n * P.C_in + c0) * P.inV;
-#pragma unroll 2
-        for (int cr = q; cr < TN; cr += KL) {
-            T b = 0;
-            if (live && c0 + cr < ce) b = sample<T, ND>(chan, voff, t.f);
-            sB[cr * LD + j] = b;
-            chan += (size_t)KL * P.inV;
+            for (int i = 0; i < NC; ++i) sIdx[wave][j][i] = live ? t.idx[i] * (unsigned)P.C_in : 0u;
+#pragma unroll
+            for (int a = 0; a < ND; ++a) sF[wave][j][a] = t.f[a];
+            sF[wave][j][3] = live ? (T)1 : (T)0;
         }
-        __syncthreads();
-        // D[m][channel] += A[m][pos] * B[pos][channel]; lane (j, q) reads row j, position ks*KL + q
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        const T* in_n = in_cl + (size_t)n * P.inV * P.C_in + cj;
+        const T* go_n = gout_cl + (size_t)n * P.outV * P.C_out;
 #pragma unroll 4
         for (int ks = 0; ks < TN / KL; ++ks) {
-            const int pp = ks * KL + q;
-            const T b = sB[j * LD + pp];
+            const int pp = ks * KL + q;                        // position of the slab this lane group works on
+            unsigned ix[NC];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(sA[(mt * TN + j) * LD + pp], b, acc[mt]);
+            for (int i = 0; i < NC; ++i) ix[i] = sIdx[wave][pp][i];
+            T f[ND];
+#pragma unroll
+            for (int a = 0; a < ND; ++a) f[a] = sF[wave][pp][a];
+            const bool lv = sF[wave][pp][3] != (T)0;
+            const T v = sample<T, ND>(in_n, ix, f);
+            const T b = (lv && chan_ok) ? v : (T)0;                                    // B[k = position][col = channel j]
+            const unsigned pg = min(p0 + (unsigned)pp, P.outV - 1);
+            const bool p_ok = p0 + (unsigned)pp < P.outV;
+            const T* grow = go_n + (size_t)pg * P.C_out;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const T a = grow[mrow[mt]];                                             // A[row = m][k = position]
+                acc[mt] = MM::mma((p_ok && m_ok[mt]) ? a : (T)0, b, acc[mt]);
+            }
         }
     }
 

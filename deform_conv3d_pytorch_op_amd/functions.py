@@ -85,15 +85,17 @@ def _geom(nd, inputs, weight, out_sizes, stride, padding, dilation, channel_per_
             list(weight.shape[2:]) + list(padding) + list(stride) + list(dilation) + [channel_per_group, group])
 
 
-def _workspace(inputs, weight, group):
+def _workspace(inputs, weight, group, out_sizes):
     L = _lib.load()
-    kV = 1
+    kV = inV = outV = 1
     for k in weight.shape[2:]:
         kV *= k
-    inV = 1
     for v in inputs.shape[2:]:
         inV *= v
-    nbytes = L.dcn_workspace_bytes(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, kV, group)
+    for v in out_sizes:
+        outV *= v
+    nbytes = L.dcn_workspace_bytes(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, outV,
+                                   kV, group)
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=inputs.device), int(nbytes)
 
 
@@ -114,7 +116,7 @@ def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channe
         _check(bias.dim() == 1 and bias.size(0) == weight.size(0), "bias size")
     inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
     output = torch.empty(out_shape, dtype=inputs.dtype, device=inputs.device)
-    ws, ws_bytes = _workspace(inputs, weight, group)
+    ws, ws_bytes = _workspace(inputs, weight, group, outs)
     fn = getattr(L, "dcn%dd_forward_%s" % (nd, _SUFFIX[inputs.dtype]))
     with torch.cuda.device(inputs.device):
         rc = fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(),
@@ -137,12 +139,12 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
     suf = _SUFFIX[inputs.dtype]
     grad_input = grad_offset = grad_weight = None
     with torch.cuda.device(inputs.device):
+        ws, ws_bytes = _workspace(inputs, weight, group, outs)
         if need_data:
             # the kernels accumulate into grad_input (as the reference's atomicAdd does) and store
             # every element of grad_offset
             grad_input = torch.zeros_like(inputs)
             grad_offset = torch.empty_like(offset)
-            ws, ws_bytes = _workspace(inputs, weight, group)
             fn = getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))
             _lib.check(fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
                           grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, _stream()))
@@ -150,7 +152,7 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
             grad_weight = torch.zeros_like(weight)          # beta = 1 accumulation, as in the reference
             fn = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
             _lib.check(fn(inputs.data_ptr(), offset.data_ptr(), grad_output.data_ptr(), grad_weight.data_ptr(),
-                          *geom, None, 0, _stream()))
+                          *geom, ws.data_ptr(), ws_bytes, _stream()))
     return grad_input, grad_offset, grad_weight
 
 

@@ -59,11 +59,11 @@ const char *dcn_arch(void);         /* the code-object target the kernels were b
 const char *dcn_last_error(void);   /* message of the last failing call on this thread ("" if none) */
 
 /* Scratch bytes any of the three calls below needs for this layer (elem_size 4 = f32, 8 = f64;
- * input_volume = input_l * input_h * input_w, kernel_volume = kernel_l * kernel_h * kernel_w).
- * The workspace holds a re-laid-out copy of the weight and, for backward_input_offset,
- * channels-last copies of one input batch and of its gradient. */
+ * input_volume = input_l * input_h * input_w, output_volume likewise, kernel_volume =
+ * kernel_l * kernel_h * kernel_w).  The workspace holds a re-laid-out copy of the weight and, for
+ * the backward calls, channels-last copies of the input batch, its gradient and grad_output. */
 size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
-                           int kernel_volume, int group);
+                           size_t output_volume, int kernel_volume, int group);
 
 /* ---- 3-D, trilinear ------------------------------------------------------------------------
  * replaces deform3d/lib/deform_conv3d_cuda.cpp:90-165 (forward), :168-262 (backward_input_offset)

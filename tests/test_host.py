@@ -31,10 +31,10 @@ def test_library_exports_every_declared_symbol():
 def test_workspace_query():
     from deform_conv3d_pytorch_op_amd import _lib
     L = _lib.load()
-    n4 = L.dcn_workspace_bytes(4, 2, 64, 64, 1000, 27, 1)
-    n8 = L.dcn_workspace_bytes(8, 2, 64, 64, 1000, 27, 1)
+    n4 = L.dcn_workspace_bytes(4, 2, 64, 64, 1000, 900, 27, 1)
+    n8 = L.dcn_workspace_bytes(8, 2, 64, 64, 1000, 900, 27, 1)
     assert n4 >= 64 * 64 * 27 * 4 + 2 * 2 * 64 * 1000 * 4 and n8 >= 64 * 64 * 27 * 8 + 2 * 2 * 64 * 1000 * 8
-    assert L.dcn_workspace_bytes(4, 2, 64, 64, 1000, 27, 0) == 0
+    assert L.dcn_workspace_bytes(4, 2, 64, 64, 1000, 900, 27, 0) == 0
 
 
 def test_argument_validation_needs_no_gpu():
