@@ -28,6 +28,16 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}     # MI355X dense matrix peaks
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 (--pmc FETCH_SIZE, then --pmc WRITE_SIZE, each scaled by
+# what the same counter reads for a plain 256 MiB device copy in the same run: 2.0 and 1.0 KiB per unit);
+# the summary with the commands is profiles/c4_deform3d_f32_fwd_bwd_kernels.md.  Only for configurations
+# that were profiled; otherwise `traffic` is null.
+MEASURED_TRAFFIC_BYTES = {
+    ("c4", "forward"): 2.603e9,
+    ("c4", "backward_input_offset"): 10.26e9,
+    ("c4", "backward_weight"): 7.363e9,
+}
+
 # name: (nd, N, C_in, C_out, in, k, stride, pad, dil, cpg, groups, offset scale / dist, dtype)
 CONFIGS = {
     "c1": (2, 2, 8, 8, 16, 3, 1, 1, 1, 8, 1, 1.5, "float64"),
@@ -68,6 +78,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c4", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic for scaling rocprof's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -159,7 +172,8 @@ def main():
     peak = PEAK_TFLOPS[spec[-1]]
     achieved = F / (kernel_ms[dominant] * 1e-3) / 1e12
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": round(achieved, 3), "peak": peak,
-                "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get((a.config, dominant)),
                 "ms": round(kernel_ms[dominant], 4),
                 "algorithmic_flops": F, "algorithmic_bytes": ab[dominant],
                 "hbm_frac_at_algorithmic_bytes": round(ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
@@ -167,21 +181,30 @@ def main():
                    "mfma_frac": round(F / (v * 1e-3) / 1e12 / peak, 4),
                    "algorithmic_GBps": round(ab[k] / (v * 1e-3) / 1e9, 1)} for k, v in kernel_ms.items()}
 
+    if a.calibrate_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)                      # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+
     # ---- CPU baseline: the oracle on a bounded sample of the same workload --------------------
     cpu = None
     if not a.no_cpu:
         from oracle import dcn_oracle as orc
-        ns = 1
+        ns = x.shape[0]
         xs, offs, gs = c["x"][:ns].contiguous(), c["off"][:ns].contiguous(), c["gout"][:ns].contiguous()
-        t0 = time.perf_counter()
-        orc.forward(xs, offs, c["w"], None, *cfg, acc64=False)
-        orc.backward(xs, offs, c["w"], gs, None, *cfg, acc64=False)
-        dt = time.perf_counter() - t0
+        reps, times = (5 if a.config in ("c4", "c5") else 9), []
+        for _ in range(reps):                  # about 5-10 s of host work at c4
+            t0 = time.perf_counter()
+            orc.forward(xs, offs, c["w"], None, *cfg, acc64=False)
+            orc.backward(xs, offs, c["w"], gs, None, *cfg, acc64=False)
+            times.append(time.perf_counter() - t0)
+        dt = sorted(times)[len(times) // 2]
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
         cpu = {"value": round(3 * F * ns / x.shape[0] / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
                "kind": "port", "seconds": round(dt, 2),
-               "sample": "%d of %d samples of %s, forward + backward once, float accumulate, OpenMP" %
-                         (ns, x.shape[0], a.config)}
+               "sample": "%d of %d samples of %s, forward + backward, median of %d runs, float accumulate, OpenMP" %
+                         (ns, x.shape[0], a.config, reps)}
 
     print(json.dumps({
         "metric": "deform conv fwd+bwd effective TFLOP/s per layer (3 dense contractions counted)",

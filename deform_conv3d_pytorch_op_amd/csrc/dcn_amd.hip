@@ -47,10 +47,11 @@ template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp)
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 // Workspace of backward_input_offset: [ re-laid-out weight | input channels-last | grad-input channels-last ]
+constexpr int TAP_PAD = 8;      // zero tap slabs behind the last group: an MFMA pass may start up to 7 taps before the end
 template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G) {
     int Mp, Cgp;
     bwd_data_weight_pad<T>(M, Cg, Mp, Cgp);
-    return align256((size_t)G * kV * Mp * Cgp * sizeof(T));
+    return align256(((size_t)G * kV + TAP_PAD) * Mp * Cgp * sizeof(T));
 }
 template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G) {
     const int M = C_out / G, Cg = C_in / G;
@@ -119,7 +120,22 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 // ---------------------------------------------------------------------------------------------
 // Halo tiling plan: block of output positions per workgroup, halo extents, channels per LDS pass.
 // Returns false when the geometry does not suit (halo too large for the staging table or LDS).
-static size_t lds_budget() { const char* e = getenv("DCN_LDS_BUDGET_KB"); return (size_t)(e ? atoi(e) : 72) * 1024; }
+// Tuning knobs (environment, read once per process):
+//   DCN_HALO_MARGIN        voxels of halo beyond the integer tap span on each side (default 2)
+//   DCN_LDS_BUDGET_KB      LDS per workgroup of the forward halo kernel (default 72: two workgroups per CU)
+//   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
+//   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
+static size_t env_kb(const char* name, int dflt) {
+    const char* e = getenv(name);
+    const int v = e ? atoi(e) : dflt;
+    return (size_t)(v > 0 ? v : dflt) * 1024;
+}
+static size_t lds_budget() { static const size_t v = env_kb("DCN_LDS_BUDGET_KB", 72); return v; }
+static size_t scatter_budget() { static const size_t v = env_kb("DCN_SCATTER_BUDGET_KB", 144); return v; }
+static bool scatter_in_lds() {
+    static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
+    return v != 0;
+}
 #define LDS_BUDGET lds_budget()
 int g_halo_margin = -1;                          // test hook: DCN_HALO_MARGIN overrides the default of 2
 
@@ -133,7 +149,7 @@ int halo_margin() {
 }
 
 template <typename T, int ND>
-bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30) {
+bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T)) {
     const int npos = WAVESH * Mma<T>::TN;       // positions per workgroup: 256 (float) or 128 (double)
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
@@ -150,11 +166,12 @@ bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30) {
         hvol *= P.hext[a];
         tiles *= P.ntile[a];
     }
-    if (hvol > (long long)WGH * NSTG) return false;
+    if (hvol > MAX_HVOL) return false;
     P.hvol = (int)hvol;
     P.hstride = ((int)hvol + 63) / 64 * 64 + 32;
     const int KL = Mma<T>::KL;
-    long long cc = (long long)(budget / ((size_t)P.hstride * sizeof(T)));
+    if (budget <= (size_t)hvol * 4) return false;
+    long long cc = (long long)((budget - (size_t)hvol * 4) / ((size_t)P.hstride * cell_bytes));
     cc = cc / KL * KL;
     const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;          // longest run of channels sharing offsets and group
     const int seg_up = (seg + KL - 1) / KL * KL;
@@ -192,8 +209,11 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     T* wt = static_cast<T*>(ws);
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     const int TN = Mma<T>::TN;
-    if (plan_halo<T, ND>(P, LDS_BUDGET)) {
-        const size_t lds = (size_t)P.cchunk * P.hstride * sizeof(T);
+    // two workgroups per CU when that still leaves 8 channels per LDS pass, else one large one
+    bool tiled = plan_halo<T, ND>(P, LDS_BUDGET);
+    if ((!tiled || P.cchunk < 8) && LDS_BUDGET < 144 * 1024) tiled = plan_halo<T, ND>(P, 144 * 1024) || tiled;
+    if (tiled) {
+        const size_t lds = (size_t)P.cchunk * P.hstride * sizeof(T) + (size_t)P.hvol * 4;
         const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
         switch (MT) {
             case 1: return launch_halo(forward_halo_kernel<T, ND, 1>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
@@ -228,47 +248,56 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     T* in_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes);
     T* gin_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes + tbytes);
     if (int rc = relayout<T>(P, w, wt, 1, s)) return rc;
+    {   // zero tap slabs behind the last group
+        const size_t used = (size_t)P.G * P.kV * P.Mp * P.Cgp, pad = (size_t)TAP_PAD * P.Mp * P.Cgp;
+        hipLaunchKernelGGL(fill_zero_kernel<T>, dim3((unsigned)((pad + 255) / 256)), dim3(256), 0, s, wt + used, pad);
+        if (int rc = check_launch("fill_zero_kernel")) return rc;
+    }
     const dim3 tgrid((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N), tblock(32, 8);
     hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
     const int TN = Mma<T>::TN;
     Params Ph = P;
-    const bool halo = plan_halo<T, ND>(Ph, LDS_BUDGET, TN) && getenv("DCN_LDS_SCATTER") != nullptr;
+    bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
+    if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
+        const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * 8);
+        if (fit >= 8) Ph.cchunk = 8;
+        else if (fit >= 4) Ph.cchunk = 4;
+        else halo = false;
+    }
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
     if (halo) {
         // grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
         T* none = nullptr;
-        switch (bwd_data_mk<T>(P.M)) {
+        switch (bwd_data_mk<T>(P.M)) {      // register-resident grad_output slab when M is small enough
             case 8: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 8>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             case 16: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 16>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             case 32: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 32>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
-            case 64: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 64>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             default: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
         }
         if (int rc = check_launch("backward_data_kernel")) return rc;
-        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * sizeof(T);
+        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4;
+        float* wmax = reinterpret_cast<float*>(gin_cl);     // the channels-last gradient buffer is free on this path
+        hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
+        if (int rc = check_launch("absmax_kernel")) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
-        switch (bwd_data_mk<T>(P.M)) {
-            case 8: return launch_halo(backward_input_halo_kernel<T, ND, 8>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
-            case 16: return launch_halo(backward_input_halo_kernel<T, ND, 16>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
-            case 32: return launch_halo(backward_input_halo_kernel<T, ND, 32>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
-            case 64: return launch_halo(backward_input_halo_kernel<T, ND, 64>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
-            default: return launch_halo(backward_input_halo_kernel<T, ND, 0>, "backward_input_halo_kernel", hgrid, lds, s, Ph, off, wt, gout, gin);
-        }
+        const int mk = bwd_data_mk<T>(P.M);
+#define DCN_SCATTER_CASE(MKV, CCHV)                                                                               \
+        if (mk == MKV && Ph.cchunk == CCHV)                                                                       \
+            return launch_halo(backward_input_halo_kernel<T, ND, MKV, CCHV>, "backward_input_halo_kernel", hgrid, \
+                               lds, s, Ph, off, wt, gout, wmax, gin);
+        DCN_SCATTER_CASE(8, 4) DCN_SCATTER_CASE(16, 4) DCN_SCATTER_CASE(32, 4) DCN_SCATTER_CASE(64, 4) DCN_SCATTER_CASE(0, 4)
+        DCN_SCATTER_CASE(8, 8) DCN_SCATTER_CASE(16, 8) DCN_SCATTER_CASE(32, 8) DCN_SCATTER_CASE(64, 8) DCN_SCATTER_CASE(0, 8)
+#undef DCN_SCATTER_CASE
+        return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }
     // halo does not fit in LDS: scatter with global atomics on the channels-last copy
     const size_t nelem = (size_t)P.N * P.C_in * P.inV;
     const unsigned fblocks = (unsigned)((nelem + 1023) / 1024 > 8192 ? 8192 : (nelem + 1023) / 1024);
     hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fblocks), dim3(256), 0, s, gin_cl, nelem);
     if (int rc = check_launch("fill_zero_kernel")) return rc;
-    switch (bwd_data_mk<T>(P.M)) {
-        case 8: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 8>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
-        case 16: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 16>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
-        case 32: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 32>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
-        case 64: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 64>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
-        default: hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff); break;
-    }
+    hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff);
     if (int rc = check_launch("backward_data_kernel")) return rc;
     hipLaunchKernelGGL(add_from_channels_last_kernel<T>, tgrid, tblock, 0, s, gin_cl, gin, P.C_in, P.inV);
     return check_launch("add_from_channels_last_kernel");

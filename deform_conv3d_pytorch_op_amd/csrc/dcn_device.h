@@ -46,7 +46,7 @@ template <> struct Mma<float> {
     __device__ static inline Acc mma(float a, float b, Acc c) {
         return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
     }
-    __device__ static inline int row(int r, int lg) { return (r >> 2) * 8 + lg * 4 + (r & 3); }
+    __host__ __device__ static constexpr int row(int r, int lg) { return (r >> 2) * 8 + lg * 4 + (r & 3); }
 };
 
 // v_mfma_f64_16x16x4_f64: A is 16x4, B is 4x16, D is 16x16.  Lane l supplies A[l%16][l/16] and
@@ -59,7 +59,7 @@ template <> struct Mma<double> {
     __device__ static inline Acc mma(double a, double b, Acc c) {
         return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
     }
-    __device__ static inline int row(int r, int lg) { return r * 4 + lg; }
+    __host__ __device__ static constexpr int row(int r, int lg) { return r * 4 + lg; }
 };
 
 template <typename T> __device__ inline typename Mma<T>::Acc acc_zero() {

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(WG) void forward_kernel(Params P, const T* __restri
 // field is handled and only the speed depends on it.
 constexpr int WGH = 512;
 constexpr int WAVESH = WGH / 64;
-constexpr int NSTG = 6;            // halo voxels staged per thread and channel: hvol <= WGH * NSTG
+constexpr int MAX_HVOL = 6144;     // halo voxels per workgroup tile (the LDS table holds one entry each)
 
 template <int ND>
 struct TileGeo {
@@ -164,45 +164,51 @@ __device__ inline bool tile_position(const Params& P, const TileGeo<ND>& tg, int
     return valid;
 }
 
-// voxel offsets (inside one channel) of the halo elements this thread stages.  Halo voxels that
-// stick out of the volume are never read by a sample, so they are simply staged from voxel 0
-// (keeps every load unconditional); slots past the halo volume are marked ~0u and skipped.
+// Table of the halo: for every halo voxel its offset inside one channel of the input, or ~0u
+// where the halo sticks out of the volume.  Built once per workgroup into LDS (hvol entries) so
+// that staging, zeroing and flushing need no per-thread index math and no registers.
 template <int ND>
-__device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsigned goff[NSTG]) {
+__device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsigned* __restrict__ sTab) {
+    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGH) {
+        int v = v0;
+        bool inb = true;
+        unsigned lin = 0;
+        int c[ND];
 #pragma unroll
-    for (int k = 0; k < NSTG; ++k) {
-        int v = threadIdx.x + WGH * k;
-        unsigned g = ~0u;
-        if (v < P.hvol) {
-            bool inb = true;
-            unsigned lin = 0;
-            int c[ND];
-#pragma unroll
-            for (int a = ND - 1; a >= 0; --a) {
-                const int s = slot<ND>(a);
-                c[a] = tg.hb[a] + v % P.hext[s];
-                v /= P.hext[s];
-                inb = inb && c[a] >= 0 && c[a] < P.in[s];
-            }
-#pragma unroll
-            for (int a = 0; a < ND; ++a) lin = lin * (unsigned)P.in[slot<ND>(a)] + (unsigned)c[a];
-            g = inb ? lin : 0u;
+        for (int a = ND - 1; a >= 0; --a) {
+            const int s = slot<ND>(a);
+            c[a] = tg.hb[a] + v % P.hext[s];
+            v /= P.hext[s];
+            inb = inb && c[a] >= 0 && c[a] < P.in[s];
         }
-        goff[k] = g;
+#pragma unroll
+        for (int a = 0; a < ND; ++a) lin = lin * (unsigned)P.in[slot<ND>(a)] + (unsigned)c[a];
+        sTab[v0] = inb ? lin : ~0u;
     }
 }
 
+// Stage `nch` channel planes of the halo.  Halo voxels outside the volume are never read by a
+// sample; they are staged from voxel 0 so that every load is unconditional.
 template <typename T>
-__device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, int nch, const unsigned goff[NSTG],
-                                  T* __restrict__ sIn) {
-    for (int c = 0; c < nch; ++c) {
-        const T* ch = chan0 + (size_t)c * P.inV;
-        T v[NSTG];
+__device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, int nch,
+                                  const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
+    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGH * 4) {
+        unsigned g[4];
 #pragma unroll
-        for (int k = 0; k < NSTG; ++k) v[k] = ch[goff[k] == ~0u ? 0u : goff[k]];     // all loads in flight together
+        for (int k = 0; k < 4; ++k) {
+            const int v = v0 + WGH * k;
+            const unsigned t = v < P.hvol ? sTab[v] : ~0u;
+            g[k] = t == ~0u ? 0u : t;
+        }
+        for (int c = 0; c < nch; ++c) {
+            const T* ch = chan0 + (size_t)c * P.inV;
+            T val[4];
 #pragma unroll
-        for (int k = 0; k < NSTG; ++k)
-            if (goff[k] != ~0u) sIn[c * P.hstride + threadIdx.x + WGH * k] = v[k];
+            for (int k = 0; k < 4; ++k) val[k] = ch[g[k]];              // four loads in flight
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (v0 + WGH * k < P.hvol) sIn[c * P.hstride + v0 + WGH * k] = val[k];
+        }
     }
 }
 
@@ -233,7 +239,8 @@ __device__ inline bool halo_corners(const Params& P, const int hb[ND], const Tap
 
 // Forward with the input halo in LDS.  Same contraction and lane roles as forward_kernel; the
 // sampled value of lane (j, q) is the MFMA B operand B[k = q][col = j].
-// grid.x = N * tiles (3-D blocks of positions), grid.y = G * mchunks; dynamic LDS = cchunk * hstride * sizeof(T).
+// grid.x = N * tiles (3-D blocks of positions), grid.y = G * mchunks;
+// dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4.
 template <typename T, int ND, int MT>
 __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __restrict__ in,
                                                            const T* __restrict__ off, const T* __restrict__ Wt,
@@ -241,7 +248,8 @@ __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sIn = reinterpret_cast<T*>(smem_raw);
+    T* sIn = reinterpret_cast<T*>(smem_raw);                                            // [cchunk][hstride]
+    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)P.cchunk * P.hstride);   // [hvol]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     const int g = blockIdx.y / P.mchunks, mchunk = blockIdx.y % P.mchunks;
@@ -254,8 +262,7 @@ __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __
     const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
-    unsigned goff[NSTG];
-    halo_table<ND>(P, tg, goff);
+    halo_table<ND>(P, tg, sTab);                   // visible after the first barrier below
 
     typename MM::Acc acc[MT];
 #pragma unroll
@@ -269,7 +276,7 @@ __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __
             const int nch = min(P.cchunk, ce - cc0);
             const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
             __syncthreads();                                               // readers of the previous chunk are done
-            halo_stage<T>(P, chan0, nch, goff, sIn);
+            halo_stage<T>(P, chan0, nch, sTab, sIn);
             __syncthreads();
             const int nsteps = (nch + KL - 1) / KL;
             T onext[ND];
@@ -632,29 +639,83 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
 }
 
 // ---------------------------------------------------------------------------------------------
+// LDS accumulation cell of the privatised scatter.  LDS float atomics (ds_add_f32) are an order
+// of magnitude slower than LDS integer atomics on gfx950, so float contributions are summed as
+// 64-bit fixed point: value * 2^e rounded to an integer and added with ds_add_u64.  The exponent
+// e is chosen per workgroup and convolution group from a bound on the largest possible term
+// (8 * max|W| * max_pos sum_m |grad_output|), leaving 2^16 terms of headroom below 2^51; the
+// integer sum is exact, so the result is rounded once when the cell is flushed.  double keeps a
+// floating cell (ds_add_f64): its 1e-10 tolerance is tighter than the fixed-point grid.
+template <typename T> struct LdsCell;
+template <> struct LdsCell<float> {
+    typedef unsigned long long type;
+    static constexpr double MAGIC = 6755399441055744.0;     // 1.5 * 2^52: low mantissa bits = integer value
+    __device__ static inline void add(type* p, float w, double gv_scaled) {
+        const double d = __builtin_fma((double)w, gv_scaled, MAGIC);
+        const long long bits = __double_as_longlong(d) - __double_as_longlong(MAGIC);
+        (void)__hip_atomic_fetch_add(p, (type)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __device__ static inline double pre(float gv, double scale) { return (double)gv * scale; }
+    __device__ static inline float value(type c, double inv_scale) { return (float)((double)(long long)c * inv_scale); }
+};
+template <> struct LdsCell<double> {
+    typedef double type;
+    __device__ static inline void add(type* p, double w, double gv) {
+        (void)__hip_atomic_fetch_add(p, w * gv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __device__ static inline double pre(double gv, double) { return gv; }
+    __device__ static inline double value(type c, double) { return c; }
+};
+
+// max |w| over a small tensor, one workgroup (used for the fixed-point exponent)
+template <typename T>
+__global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restrict__ out) {
+    __shared__ float red[1024];
+    float m = 0.f;
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf((float)w[i]));
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int sft = blockDim.x / 2; sft > 0; sft >>= 1) {
+        if ((int)threadIdx.x < sft) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + sft]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0];
+}
+
+// ---------------------------------------------------------------------------------------------
 // Backward to input with the scatter privatised in LDS (col2im_input of the reference,
 // deform3d kernel.cu:229-296 / deform2d_double kernel.cu:201-238, fed by the grad-column GEMM of
 // deform3d/lib/deform_conv3d_cuda.cpp:213-220).
 //
-// Same halo tiling as forward_halo_kernel, but the LDS planes hold the partial grad-input of
-// `cchunk` (<= TN) channels over the halo of the workgroup's position block.  Per tap the
-// grad-column tile gcol[c][pos] (rows = the chunk's channels, lanes = positions) comes out of
-// MFMA; each lane adds its values to the 8 (4) corners with LDS float atomics
-// ((w_l*w_h*w_w)*gcol as in the reference).  After the 27 taps the planes are added to
-// grad_input with one hardware atomic per touched halo voxel -- about 1/30 of the global
-// atomics of a direct scatter.  Samples that reach past the halo use global atomics directly.
+// Same halo tiling as forward_halo_kernel, but the LDS planes hold the partial grad-input of CCH
+// channels over the halo of the workgroup's position block (cells: see LdsCell).  The rows of
+// one MFMA tile are (tap, channel) pairs -- TP = TN / CCH taps of the CCH channels -- so a pass
+// of MK MFMAs yields the grad-column values gcol[c][tap][pos] of TP taps at once with lanes
+// along positions.  Each lane then walks its registers: per tap it derives the corner indices
+// and weights of its position and adds (w_l*w_h*w_w)*gcol to the 8 (4) corners with LDS integer
+// atomics.  After all taps the planes are added to grad_input with one hardware float atomic per
+// touched halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that
+// reach past the halo use global atomics directly.
 // MK > 0: the wavefront's grad_output slab (MK reduction steps = M rounded up / KL) stays in
-// registers for the whole tile; MK == 0: it is re-read per tap (any M).
-// grid.x = N * tiles, grid.y = DG; dynamic LDS = cchunk * hstride * sizeof(T).
-template <typename T, int ND, int MK>
+// registers for the whole tile; MK == 0: it is re-read per pass (any M).
+// grid.x = N * tiles, grid.y = DG; dynamic LDS = CCH * hstride * 8 + hvol * 4 bytes.
+template <typename T, int ND, int MK, int CCH>
 __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
                                                                   const T* __restrict__ gout,
+                                                                  const float* __restrict__ wmax,
                                                                   T* __restrict__ gin) {
     using MM = Mma<T>;
+    using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
+    constexpr int TP = TN / CCH;                        // taps per MFMA pass
+    constexpr int RPS = (MM::row(1, 0) - MM::row(0, 0) == 1) ? 4 : CCH / 4;   // registers that share a tap
+    constexpr int NS = NACC / RPS;                      // tap slots per lane and pass
+    static_assert(TN % CCH == 0 && CCH % 4 == 0 && NACC % RPS == 0, "unsupported channel chunk");
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sG = reinterpret_cast<T*>(smem_raw);
+    Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
+    unsigned* sTab = reinterpret_cast<unsigned*>(sG + (size_t)CCH * P.hstride);         // [hvol]
+    __shared__ float sRed[WAVESH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     const int dg = blockIdx.y;
@@ -667,68 +728,82 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
-    unsigned goff[NSTG];
-    halo_table<ND>(P, tg, goff);
+    halo_table<ND>(P, tg, sTab);                   // visible after the first barrier below
 
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+    // this lane's row of the A operand: (tap slot, channel) = (j / CCH, j % CCH)
+    const int a_tl = j / CCH, a_c = j % CCH;
 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
         const T* gq0 = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + pos;
         T breg[MK > 0 ? MK : 1];
+        float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
         if constexpr (MK > 0) {
 #pragma unroll
-            for (int k = 0; k < MK; ++k)
+            for (int k = 0; k < MK; ++k) {
                 breg[k] = (valid && k * KL + q < P.M) ? gq0[(size_t)k * KL * P.outV] : (T)0;
+                sabs += fabsf((float)breg[k]);
+            }
+        } else {
+            const T* gq = gq0;
+            for (int m0 = 0; m0 < P.M; m0 += KL) {
+                if (valid && m0 + q < P.M) sabs += fabsf((float)*gq);
+                gq += (size_t)KL * P.outV;
+            }
         }
-        for (int cc0 = rb; cc0 < re; cc0 += P.cchunk) {
-            const int nch = min(P.cchunk, re - cc0);
+        // fixed-point exponent of this (workgroup, convolution group): terms are bounded by
+        // 8 * max|W| * max_pos sum_m |grad_output|
+#pragma unroll
+        for (int sh = TN; sh < 64; sh <<= 1) sabs += __shfl_xor(sabs, sh);
+#pragma unroll
+        for (int sh = 1; sh < TN; sh <<= 1) sabs = fmaxf(sabs, __shfl_xor(sabs, sh));
+        __syncthreads();
+        if (lane == 0) sRed[wave] = sabs;
+        __syncthreads();
+        float smax = 0.f;
+#pragma unroll
+        for (int w8 = 0; w8 < WAVESH; ++w8) smax = fmaxf(smax, sRed[w8]);
+        int ex = 0;
+        const float bound = 8.f * wmax[0] * smax;
+        if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
+        const double scale = ldexp(1.0, 34 - ex), inv_scale = ldexp(1.0, ex - 34);
+
+        for (int cc0 = rb; cc0 < re; cc0 += CCH) {
+            const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
-#pragma unroll
-                for (int k = 0; k < NSTG; ++k)
-                    if (goff[k] != ~0u) sG[c * P.hstride + threadIdx.x + WGH * k] = 0;
+                for (int v = threadIdx.x; v < P.hvol; v += WGH) sG[c * P.hstride + v] = 0;      // all-zero bits in either cell type
             __syncthreads();
 
-            T onext[ND];
-            load_offsets<T, ND>(P, off_dg, pos, onext);
-            for (int tap = 0; tap < P.kV; ++tap) {
-                int kk[ND], kd[ND];
-                decode_tap<ND>(P, tap, kk);
+            for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
+                // offsets of this lane's tap slots travel while the MFMA pass runs
+                T ofs[NS][ND];
+                int tap_s[NS];
 #pragma unroll
-                for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
-                T ocur[ND];
-#pragma unroll
-                for (int a = 0; a < ND; ++a) ocur[a] = onext[a];
-                if (tap + 1 < P.kV) load_offsets<T, ND>(P, off_dg + (size_t)(tap + 1) * ND * P.outV, pos, onext);
-                TapGeo<T, ND> t;
-                tap_setup<T, ND>(P, ocur, ib, kd, t);
-                const bool live = valid && t.inside;
-                if (!__any(live)) continue;
-                unsigned lidx[NC];
-                const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
-                const bool near = live && in_halo, far = live && !in_halo;
-                T cw[NC];
-                if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
-                    const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
-                    cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
-                    cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
-                } else {
-                    const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                    cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                for (int ts = 0; ts < NS; ++ts) {
+                    tap_s[ts] = tap0 + MM::row(ts * RPS, q) / CCH;
+                    const int tl = min(tap_s[ts], P.kV - 1);
+                    load_offsets<T, ND>(P, off_dg + (size_t)tl * ND * P.outV, pos, ofs[ts]);
                 }
-                // grad-column tile: rows = channels cc0 + i, columns = this wavefront's positions
+                // grad-column tile: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past the
+                // last one read zero padding (or rows that are ignored below)
                 typename MM::Acc d = acc_zero<T>();
-                const T* wa = Wt + (((size_t)g * P.kV + tap) * P.Mp + q) * P.Cgp + (cc0 - g * P.Cg) + j;
+                const T* wa = Wt + (((size_t)g * P.kV + tap0 + a_tl) * P.Mp + q) * P.Cgp + (cc0 - g * P.Cg) + a_c;
                 if constexpr (MK > 0) {
-                    // all weight loads of the tile are issued before the first MFMA needs one
-                    T areg[MK];
+                    // weight loads in batches of 16, each batch issued before its MFMAs need it
+                    constexpr int AB = MK < 16 ? MK : 16;
 #pragma unroll
-                    for (int k = 0; k < MK; ++k) areg[k] = wa[(size_t)k * KL * P.Cgp];
-                    __builtin_amdgcn_sched_barrier(0);      // keep the loads batched ahead of the MFMA chain
+                    for (int k0 = 0; k0 < MK; k0 += AB) {
+                        T areg[AB];
 #pragma unroll
-                    for (int k = 0; k < MK; ++k) d = MM::mma(areg[k], breg[k], d);
+                        for (int k = 0; k < AB; ++k) areg[k] = wa[(size_t)(k0 + k) * KL * P.Cgp];
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) d = MM::mma(areg[k], breg[k0 + k], d);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 } else {
                     const T* gq = gq0;
                     for (int m0 = 0; m0 < P.M; m0 += KL) {
@@ -739,31 +814,56 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     }
                 }
 #pragma unroll
-                for (int r = 0; r < NACC; ++r) {
-                    const int cl = MM::row(r, q);
-                    if (cl < nch) {
-                        const T gv = d[r];
-                        if (near) {
-                            T* plane = sG + cl * P.hstride;
+                for (int ts = 0; ts < NS; ++ts) {
+                    const int tap = tap_s[ts];
+                    int kk[ND], kd[ND];
+                    decode_tap<ND>(P, min(tap, P.kV - 1), kk);
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) lds_atomic_add(plane + lidx[i], cw[i] * gv);
-                        } else if (far) {
+                    for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+                    TapGeo<T, ND> t;
+                    tap_setup<T, ND>(P, ofs[ts], ib, kd, t);
+                    const bool live = valid && t.inside && tap < P.kV;
+                    if (!live) continue;
+                    unsigned lidx[NC];
+                    const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+                    T cw[NC];
+                    if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
+                        const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                        cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                        cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+                    } else {
+                        const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                        cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                    }
+#pragma unroll
+                    for (int rr = 0; rr < RPS; ++rr) {
+                        const int r = ts * RPS + rr;
+                        const int cl = MM::row(r, q) % CCH;
+                        if (cl >= nch) continue;
+                        const T gv = d[r];
+                        if (in_halo) {
+                            Cell* plane = sG + cl * P.hstride;
+                            const double gs = LdsCell<T>::pre(gv, scale);
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+                        } else {
                             T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
 #pragma unroll
                             for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
                         }
                     }
+                    __builtin_amdgcn_sched_barrier(0);      // one tap slot at a time: keeps the live register set small
                 }
             }
             __syncthreads();                        // all LDS adds of this chunk have landed
-            for (int c = 0; c < nch; ++c) {
-                T* gc = gin + ((size_t)n * P.C_in + cc0 + c) * P.inV;
-#pragma unroll
-                for (int k = 0; k < NSTG; ++k)
-                    if (goff[k] != ~0u) {
-                        const T v = sG[c * P.hstride + threadIdx.x + WGH * k];
-                        if (v != (T)0) atomic_add(gc + goff[k], v);
-                    }
+            for (int v = threadIdx.x; v < P.hvol; v += WGH) {
+                const unsigned gv = sTab[v];
+                if (gv == ~0u) continue;            // halo cell outside the volume: never touched
+                for (int c = 0; c < nch; ++c) {
+                    const Cell cell = sG[c * P.hstride + v];
+                    if (cell != (Cell)0)
+                        atomic_add(gin + ((size_t)n * P.C_in + cc0 + c) * P.inV + gv, (T)LdsCell<T>::value(cell, inv_scale));
+                }
             }
         }
     }

@@ -1,0 +1,34 @@
+"""Runs the small parity cases again with the library's tuning knobs forced to the corner
+settings, each in a process of its own (the knobs are read once per process):
+
+  DCN_HALO_MARGIN=0    almost every sample reaches past the LDS halo -> global fallback paths
+  DCN_HALO_MARGIN=50   the halo never fits -> kernels that do not use LDS tiling at all
+  DCN_SCATTER=global   grad-input through global atomics on the channels-last copy
+  DCN_LDS_BUDGET_KB / DCN_SCATTER_BUDGET_KB small -> smallest channel chunks
+"""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+SETTINGS = [
+    {"DCN_HALO_MARGIN": "0"},
+    {"DCN_HALO_MARGIN": "50"},
+    {"DCN_SCATTER": "global"},
+    {"DCN_LDS_BUDGET_KB": "16", "DCN_SCATTER_BUDGET_KB": "72"},
+]
+
+
+@pytest.mark.parametrize("extra", SETTINGS, ids=lambda e: ",".join("%s=%s" % kv for kv in e.items()))
+def test_small_cases_under_knob(extra):
+    print("knobs", extra, flush=True)
+    env = dict(os.environ)
+    env.update(extra)
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.join(ROOT, "tests", "test_gpu_parity.py"), "-q", "-x",
+                        "-m", "gpu", "-k", "small_cases or golden", "--timeout", "120", "--timeout-method", "thread"],
+                       cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:]
