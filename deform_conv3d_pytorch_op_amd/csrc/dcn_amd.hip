@@ -125,6 +125,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_LDS_BUDGET_KB      LDS per workgroup of the forward halo kernel (default 72: two workgroups per CU)
 //   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
+//   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
 static size_t env_kb(const char* name, int dflt) {
     const char* e = getenv(name);
     const int v = e ? atoi(e) : dflt;
@@ -132,6 +133,10 @@ static size_t env_kb(const char* name, int dflt) {
 }
 static size_t lds_budget() { static const size_t v = env_kb("DCN_LDS_BUDGET_KB", 72); return v; }
 static size_t scatter_budget() { static const size_t v = env_kb("DCN_SCATTER_BUDGET_KB", 144); return v; }
+static bool fused_coord() {
+    static const int v = [] { const char* e = getenv("DCN_COORD"); return (e && strcmp(e, "separate") == 0) ? 0 : 1; }();
+    return v != 0;
+}
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
     return v != 0;
@@ -253,11 +258,32 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         hipLaunchKernelGGL(fill_zero_kernel<T>, dim3((unsigned)((pad + 255) / 256)), dim3(256), 0, s, wt + used, pad);
         if (int rc = check_launch("fill_zero_kernel")) return rc;
     }
+    const int TN = Mma<T>::TN;
+    const int mk = bwd_data_mk<T>(P.M);
+    float* wmax = reinterpret_cast<float*>(gin_cl);     // the channels-last gradient buffer is free on the LDS paths
     const dim3 tgrid((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N), tblock(32, 8);
+
+    // 1) one kernel: scatter privatised in LDS + coordinate gradient from an LDS input halo
+    Params Ph = P;
+    if (scatter_in_lds() && fused_coord() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T)) &&
+        (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4) {
+        Ph.cchunk = 4;
+        const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4;
+        hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
+        if (int rc = check_launch("absmax_kernel")) return rc;
+        const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
+#define DCN_FUSED_CASE(MKV)                                                                                       \
+        if (mk == MKV)                                                                                            \
+            return launch_halo(backward_input_halo_kernel<T, ND, MKV, 4, true>, "backward_input_halo_kernel",     \
+                               hgrid, lds, s, Ph, in, off, wt, gout, wmax, gin, goff);
+        DCN_FUSED_CASE(8) DCN_FUSED_CASE(16) DCN_FUSED_CASE(32) DCN_FUSED_CASE(64) DCN_FUSED_CASE(0)
+#undef DCN_FUSED_CASE
+    }
+
+    // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
     hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
-    const int TN = Mma<T>::TN;
-    Params Ph = P;
+    Ph = P;
     bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
     if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
         const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * 8);
@@ -268,9 +294,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
     if (halo) {
-        // grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
         T* none = nullptr;
-        switch (bwd_data_mk<T>(P.M)) {      // register-resident grad_output slab when M is small enough
+        switch (mk) {      // register-resident grad_output slab when M is small enough
             case 8: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 8>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             case 16: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 16>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             case 32: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 32>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
@@ -278,15 +303,14 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         }
         if (int rc = check_launch("backward_data_kernel")) return rc;
         const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4;
-        float* wmax = reinterpret_cast<float*>(gin_cl);     // the channels-last gradient buffer is free on this path
         hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
         if (int rc = check_launch("absmax_kernel")) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
-        const int mk = bwd_data_mk<T>(P.M);
+        T* nogoff = nullptr;
 #define DCN_SCATTER_CASE(MKV, CCHV)                                                                               \
         if (mk == MKV && Ph.cchunk == CCHV)                                                                       \
-            return launch_halo(backward_input_halo_kernel<T, ND, MKV, CCHV>, "backward_input_halo_kernel", hgrid, \
-                               lds, s, Ph, off, wt, gout, wmax, gin);
+            return launch_halo(backward_input_halo_kernel<T, ND, MKV, CCHV, false>, "backward_input_halo_kernel", \
+                               hgrid, lds, s, Ph, in, off, wt, gout, wmax, gin, nogoff);
         DCN_SCATTER_CASE(8, 4) DCN_SCATTER_CASE(16, 4) DCN_SCATTER_CASE(32, 4) DCN_SCATTER_CASE(64, 4) DCN_SCATTER_CASE(0, 4)
         DCN_SCATTER_CASE(8, 8) DCN_SCATTER_CASE(16, 8) DCN_SCATTER_CASE(32, 8) DCN_SCATTER_CASE(64, 8) DCN_SCATTER_CASE(0, 8)
 #undef DCN_SCATTER_CASE

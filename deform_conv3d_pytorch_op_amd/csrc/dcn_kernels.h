@@ -699,12 +699,19 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // MK > 0: the wavefront's grad_output slab (MK reduction steps = M rounded up / KL) stays in
 // registers for the whole tile; MK == 0: it is re-read per pass (any M).
 // grid.x = N * tiles, grid.y = DG; dynamic LDS = CCH * hstride * 8 + hvol * 4 bytes.
-template <typename T, int ND, int MK, int CCH>
-__global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ off,
+// COORD = true additionally stages the same CCH input channels over the halo (float planes) and
+// computes grad_offset in the same pass over the grad-column values (col2im_offset of the
+// reference, deform3d kernel.cu:386-483 incl. the out-of-range branches :470-481, 2-D
+// deform2d_double kernel.cu:309-366): per (tap, position) the derivative of the interpolation
+// along each axis times gcol, summed over the chunk's channels, accumulated into grad_offset
+// chunk after chunk (the first chunk stores).  dynamic LDS then adds CCH * hstride * sizeof(T).
+template <typename T, int ND, int MK, int CCH, bool COORD>
+__global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
+                                                                  const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
                                                                   const T* __restrict__ gout,
                                                                   const float* __restrict__ wmax,
-                                                                  T* __restrict__ gin) {
+                                                                  T* __restrict__ gin, T* __restrict__ goff) {
     using MM = Mma<T>;
     using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
@@ -714,7 +721,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     static_assert(TN % CCH == 0 && CCH % 4 == 0 && NACC % RPS == 0, "unsupported channel chunk");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
-    unsigned* sTab = reinterpret_cast<unsigned*>(sG + (size_t)CCH * P.hstride);         // [hvol]
+    T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * P.hstride);                        // [CCH][hstride] if COORD
+    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * P.hstride : 0));   // [hvol]
     __shared__ float sRed[WAVESH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
@@ -732,8 +740,11 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+    T* goff_dg = goff + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+    bool first_chunk = true;                        // grad_offset: the first channel chunk stores, later ones add
     // this lane's row of the A operand: (tap slot, channel) = (j / CCH, j % CCH)
     const int a_tl = j / CCH, a_c = j % CCH;
+    const unsigned a_off = ((unsigned)a_tl * P.Mp + q) * P.Cgp + a_c;      // lane offset inside a tap group's weight slabs
 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
@@ -741,9 +752,14 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
         T breg[MK > 0 ? MK : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
         if constexpr (MK > 0) {
+            // running pointer, made opaque so that the MK addresses are not hoisted out of the group
+            // loop and kept alive (they would cost 2*MK registers for the whole kernel)
+            const T* gp = gq0;
+            asm volatile("" : "+v"(gp));
 #pragma unroll
             for (int k = 0; k < MK; ++k) {
-                breg[k] = (valid && k * KL + q < P.M) ? gq0[(size_t)k * KL * P.outV] : (T)0;
+                breg[k] = (valid && k * KL + q < P.M) ? *gp : (T)0;
+                gp += (size_t)KL * P.outV;
                 sabs += fabsf((float)breg[k]);
             }
         } else {
@@ -775,6 +791,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
                 for (int v = threadIdx.x; v < P.hvol; v += WGH) sG[c * P.hstride + v] = 0;      // all-zero bits in either cell type
+            if constexpr (COORD) halo_stage<T>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
 
             for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
@@ -790,7 +807,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                 // grad-column tile: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past the
                 // last one read zero padding (or rows that are ignored below)
                 typename MM::Acc d = acc_zero<T>();
-                const T* wa = Wt + (((size_t)g * P.kV + tap0 + a_tl) * P.Mp + q) * P.Cgp + (cc0 - g * P.Cg) + a_c;
+                // wave-uniform slab pointer + one 32-bit lane offset: the loads need no per-load address registers
+                const T* wu = Wt + (((size_t)g * P.kV + tap0) * P.Mp) * P.Cgp + (cc0 - g * P.Cg);
                 if constexpr (MK > 0) {
                     // weight loads in batches of 16, each batch issued before its MFMAs need it
                     constexpr int AB = MK < 16 ? MK : 16;
@@ -798,7 +816,10 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     for (int k0 = 0; k0 < MK; k0 += AB) {
                         T areg[AB];
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) areg[k] = wa[(size_t)(k0 + k) * KL * P.Cgp];
+                        for (int k = 0; k < AB; ++k) {
+                            areg[k] = wu[a_off];
+                            wu += (size_t)KL * P.Cgp;
+                        }
                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                         for (int k = 0; k < AB; ++k) d = MM::mma(areg[k], breg[k0 + k], d);
@@ -808,8 +829,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     const T* gq = gq0;
                     for (int m0 = 0; m0 < P.M; m0 += KL) {
                         const T b = (valid && m0 + q < P.M) ? *gq : (T)0;
-                        d = MM::mma(*wa, b, d);
-                        wa += (size_t)KL * P.Cgp;
+                        d = MM::mma(wu[a_off], b, d);
+                        wu += (size_t)KL * P.Cgp;
                         gq += (size_t)KL * P.outV;
                     }
                 }
@@ -822,39 +843,104 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
                     TapGeo<T, ND> t;
                     tap_setup<T, ND>(P, ofs[ts], ib, kd, t);
-                    const bool live = valid && t.inside && tap < P.kV;
-                    if (!live) continue;
-                    unsigned lidx[NC];
-                    const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
-                    T cw[NC];
-                    if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
-                        const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
-                        cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
-                        cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
-                    } else {
-                        const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                        cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
-                    }
+                    const bool slot_ok = valid && tap < P.kV;
+                    const bool live = slot_ok && t.inside;
+                    T ga[ND];
 #pragma unroll
-                    for (int rr = 0; rr < RPS; ++rr) {
-                        const int r = ts * RPS + rr;
-                        const int cl = MM::row(r, q) % CCH;
-                        if (cl >= nch) continue;
-                        const T gv = d[r];
-                        if (in_halo) {
-                            Cell* plane = sG + cl * P.hstride;
-                            const double gs = LdsCell<T>::pre(gv, scale);
-#pragma unroll
-                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+                    for (int a = 0; a < ND; ++a) ga[a] = 0;
+                    if (live) {
+                        unsigned lidx[NC];
+                        const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+                        T cw[NC];
+                        if constexpr (ND == 3) {   // multiplied in the reference's order (w_l * w_h * w_w)
+                            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                            cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                            cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
                         } else {
-                            T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
+                            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                            cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                        }
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
+                        for (int rr = 0; rr < RPS; ++rr) {
+                            const int r = ts * RPS + rr;
+                            const int cl = MM::row(r, q) % CCH;
+                            if (cl >= nch) continue;
+                            const T gv = d[r];
+                            T v[NC];
+                            if (in_halo) {
+                                Cell* plane = sG + cl * P.hstride;
+                                const double gs = LdsCell<T>::pre(gv, scale);
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+                                if constexpr (COORD) {
+                                    const T* ip = sIn + cl * P.hstride;
+#pragma unroll
+                                    for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
+                                }
+                            } else {
+                                T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
+                                if constexpr (COORD) {
+                                    const T* ic = in + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
+#pragma unroll
+                                    for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
+                                }
+                            }
+                            if constexpr (COORD) {
+                                if constexpr (ND == 3) {
+                                    const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh,
+                                            fw = t.f[2], gw = (T)1 - fw;
+                                    ga[0] += gv * (((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
+                                                   ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh);
+                                    ga[1] += gv * (((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
+                                                   ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl);
+                                    ga[2] += gv * (((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                                   ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl);
+                                } else {
+                                    const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                                    ga[0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
+                                    ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
+                                }
+                            }
+                        }
+                    } else if (COORD && ND == 3 && slot_ok) {
+                        // out-of-range sample: +-|gcol| per axis; h and w are compared with the LENGTH extent
+                        const T len = (T)P.in[0];
+                        T sg[ND];
+#pragma unroll
+                        for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= len) ? (T)1 : (T)0);
+#pragma unroll
+                        for (int rr = 0; rr < RPS; ++rr) {
+                            const int r = ts * RPS + rr;
+                            if (MM::row(r, q) % CCH >= nch) continue;
+                            const T av = d[r] > 0 ? d[r] : -d[r];
+#pragma unroll
+                            for (int a = 0; a < ND; ++a) ga[a] += sg[a] * av;
+                        }
+                    }
+                    if constexpr (COORD) {
+                        // channels of one (tap, position) that sit in other lane groups are summed in
+                        if constexpr (RPS < CCH) {
+#pragma unroll
+                            for (int a = 0; a < ND; ++a)
+#pragma unroll
+                                for (int sh = TN; sh < TN * (CCH / RPS); sh <<= 1) ga[a] += __shfl_xor(ga[a], sh);
+                        }
+                        const bool owner = (RPS == CCH) || (q % (CCH / RPS)) == 0;
+                        if (slot_ok && owner) {
+                            T* gp = goff_dg + (size_t)tap * ND * P.outV + pos;
+#pragma unroll
+                            for (int a = 0; a < ND; ++a) {
+                                if (first_chunk) gp[(size_t)a * P.outV] = ga[a];
+                                else gp[(size_t)a * P.outV] += ga[a];
+                            }
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);      // one tap slot at a time: keeps the live register set small
                 }
             }
+            first_chunk = false;
             __syncthreads();                        // all LDS adds of this chunk have landed
             for (int v = threadIdx.x; v < P.hvol; v += WGH) {
                 const unsigned gv = sTab[v];
