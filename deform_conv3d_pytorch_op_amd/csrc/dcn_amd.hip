@@ -39,14 +39,16 @@ template <typename T> int bwd_data_mk(int M) {
     return 0;
 }
 template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp) {
-    const int mk = bwd_data_mk<T>(M) * Mma<T>::KL;
-    Mp = M + Mma<T>::KL;
+    // rows: reduction steps are consumed in batches of 8; the coordinate kernel reads up to KL rows further
+    const int KL = Mma<T>::KL;
+    const int steps = ((M + KL - 1) / KL + 7) / 8 * 8;
+    Mp = steps * KL + KL;
+    const int mk = bwd_data_mk<T>(M) * KL;
     if (mk > Mp) Mp = mk;
     Cgp = Cg + Mma<T>::TN;
 }
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
-// Workspace of backward_input_offset: [ re-laid-out weight | input channels-last | grad-input channels-last ]
 constexpr int TAP_PAD = 8;      // zero tap slabs behind the last group: an MFMA pass may start up to 7 taps before the end
 template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G) {
     int Mp, Cgp;
@@ -136,6 +138,17 @@ static size_t scatter_budget() { static const size_t v = env_kb("DCN_SCATTER_BUD
 static bool fused_coord() {
     static const int v = [] { const char* e = getenv("DCN_COORD"); return (e && strcmp(e, "separate") == 0) ? 0 : 1; }();
     return v != 0;
+}
+static int cu_count() {
+    static const int v = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        return n;
+    }();
+    return v;
 }
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
@@ -271,13 +284,27 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4;
         hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
         if (int rc = check_launch("absmax_kernel")) return rc;
-        const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
-#define DCN_FUSED_CASE(MKV)                                                                                       \
-        if (mk == MKV)                                                                                            \
-            return launch_halo(backward_input_halo_kernel<T, ND, MKV, 4, true>, "backward_input_halo_kernel",     \
-                               hgrid, lds, s, Ph, in, off, wt, gout, wmax, gin, goff);
-        DCN_FUSED_CASE(8) DCN_FUSED_CASE(16) DCN_FUSED_CASE(32) DCN_FUSED_CASE(64) DCN_FUSED_CASE(0)
-#undef DCN_FUSED_CASE
+        // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
+        // wastes least of the last round (one workgroup per CU at this LDS size)
+        const int nchunks = ((P.cpg < P.Cg ? P.cpg : P.Cg) + 3) / 4;
+        const long long items = (long long)Ph.N * Ph.tiles * Ph.DG;
+        const int cus = cu_count();
+        int csplit = 1;
+        double best = 1e30;
+        for (int cs = 1; cs <= 4 && cs <= nchunks; cs *= 2) {
+            const double rounds = (double)((items * cs + cus - 1) / cus) / cs;
+            if (rounds < best * 0.97) { best = rounds; csplit = cs; }
+        }
+        if (const char* e = getenv("DCN_CSPLIT")) csplit = atoi(e) > 0 ? atoi(e) : csplit;
+        if (csplit > 1) {
+            const size_t nel = (size_t)P.N * P.DG * P.kV * ND * P.outV;
+            const unsigned fb = (unsigned)((nel + 1023) / 1024 > 8192 ? 8192 : (nel + 1023) / 1024);
+            hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fb), dim3(256), 0, s, goff, nel);
+            if (int rc = check_launch("fill_zero_kernel")) return rc;
+        }
+        const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG, (unsigned)csplit);
+        return launch_halo(backward_input_halo_kernel<T, ND, 4, true>, "backward_input_halo_kernel", hgrid, lds, s, Ph,
+                           in, off, wt, gout, wmax, gin, goff);
     }
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
@@ -307,13 +334,12 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         if (int rc = check_launch("absmax_kernel")) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
         T* nogoff = nullptr;
-#define DCN_SCATTER_CASE(MKV, CCHV)                                                                               \
-        if (mk == MKV && Ph.cchunk == CCHV)                                                                       \
-            return launch_halo(backward_input_halo_kernel<T, ND, MKV, CCHV, false>, "backward_input_halo_kernel", \
-                               hgrid, lds, s, Ph, in, off, wt, gout, wmax, gin, nogoff);
-        DCN_SCATTER_CASE(8, 4) DCN_SCATTER_CASE(16, 4) DCN_SCATTER_CASE(32, 4) DCN_SCATTER_CASE(64, 4) DCN_SCATTER_CASE(0, 4)
-        DCN_SCATTER_CASE(8, 8) DCN_SCATTER_CASE(16, 8) DCN_SCATTER_CASE(32, 8) DCN_SCATTER_CASE(64, 8) DCN_SCATTER_CASE(0, 8)
-#undef DCN_SCATTER_CASE
+        if (Ph.cchunk == 8)
+            return launch_halo(backward_input_halo_kernel<T, ND, 8, false>, "backward_input_halo_kernel", hgrid, lds, s,
+                               Ph, in, off, wt, gout, wmax, gin, nogoff);
+        if (Ph.cchunk == 4)
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, false>, "backward_input_halo_kernel", hgrid, lds, s,
+                               Ph, in, off, wt, gout, wmax, gin, nogoff);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }
     // halo does not fit in LDS: scatter with global atomics on the channels-last copy

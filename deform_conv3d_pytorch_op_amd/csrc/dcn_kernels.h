@@ -696,8 +696,6 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // atomics.  After all taps the planes are added to grad_input with one hardware float atomic per
 // touched halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that
 // reach past the halo use global atomics directly.
-// MK > 0: the wavefront's grad_output slab (MK reduction steps = M rounded up / KL) stays in
-// registers for the whole tile; MK == 0: it is re-read per pass (any M).
 // grid.x = N * tiles, grid.y = DG; dynamic LDS = CCH * hstride * 8 + hvol * 4 bytes.
 // COORD = true additionally stages the same CCH input channels over the halo (float planes) and
 // computes grad_offset in the same pass over the grad-column values (col2im_offset of the
@@ -705,7 +703,7 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // deform2d_double kernel.cu:309-366): per (tap, position) the derivative of the interpolation
 // along each axis times gcol, summed over the chunk's channels, accumulated into grad_offset
 // chunk after chunk (the first chunk stores).  dynamic LDS then adds CCH * hstride * sizeof(T).
-template <typename T, int ND, int MK, int CCH, bool COORD>
+template <typename T, int ND, int CCH, bool COORD>
 __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
@@ -727,6 +725,10 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     const int dg = blockIdx.y;
+    // gridDim.z workgroups share one (tile, deformable group): workgroup z takes every gridDim.z-th
+    // channel chunk (finer work items shorten the last, partly filled round of workgroups).  Their
+    // grad_offset contributions then meet through float atomics on a zero-filled buffer.
+    const int csplit = gridDim.z, cz = blockIdx.z;
 
     TileGeo<ND> tg;
     tile_decode<ND>(P, blockIdx.x, tg);
@@ -741,7 +743,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
     T* goff_dg = goff + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
-    bool first_chunk = true;                        // grad_offset: the first channel chunk stores, later ones add
+    bool first_chunk = true;                        // grad_offset (csplit == 1): the first channel chunk stores, later ones add
+    int chunk_no = 0;
     // this lane's row of the A operand: (tap slot, channel) = (j / CCH, j % CCH)
     const int a_tl = j / CCH, a_c = j % CCH;
     const unsigned a_off = ((unsigned)a_tl * P.Mp + q) * P.Cgp + a_c;      // lane offset inside a tap group's weight slabs
@@ -749,20 +752,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
         const T* gq0 = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + pos;
-        T breg[MK > 0 ? MK : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
-        if constexpr (MK > 0) {
-            // running pointer, made opaque so that the MK addresses are not hoisted out of the group
-            // loop and kept alive (they would cost 2*MK registers for the whole kernel)
-            const T* gp = gq0;
-            asm volatile("" : "+v"(gp));
-#pragma unroll
-            for (int k = 0; k < MK; ++k) {
-                breg[k] = (valid && k * KL + q < P.M) ? *gp : (T)0;
-                gp += (size_t)KL * P.outV;
-                sabs += fabsf((float)breg[k]);
-            }
-        } else {
+        {
             const T* gq = gq0;
             for (int m0 = 0; m0 < P.M; m0 += KL) {
                 if (valid && m0 + q < P.M) sabs += fabsf((float)*gq);
@@ -787,6 +778,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
         const double scale = ldexp(1.0, 34 - ex), inv_scale = ldexp(1.0, ex - 34);
 
         for (int cc0 = rb; cc0 < re; cc0 += CCH) {
+            if ((chunk_no++) % csplit != cz) continue;          // another workgroup's chunk (uniform)
             const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
@@ -807,35 +799,49 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                 // grad-column tile: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past the
                 // last one read zero padding (or rows that are ignored below)
                 typename MM::Acc d = acc_zero<T>();
-                // wave-uniform slab pointer + one 32-bit lane offset: the loads need no per-load address registers
-                const T* wu = Wt + (((size_t)g * P.kV + tap0) * P.Mp) * P.Cgp + (cc0 - g * P.Cg);
-                if constexpr (MK > 0) {
-                    // weight loads in batches of 16, each batch issued before its MFMAs need it
-                    constexpr int AB = MK < 16 ? MK : 16;
-#pragma unroll
-                    for (int k0 = 0; k0 < MK; k0 += AB) {
-                        T areg[AB];
+                // operands in batches of AB reduction steps: all loads of a batch are issued before its
+                // MFMAs need them; a rolled loop with two running pointers keeps the address state small
+                {
+                    constexpr int AB = 8;
+                    const T* wp = Wt + (((size_t)g * P.kV + tap0) * P.Mp) * P.Cgp + (cc0 - g * P.Cg) + a_off;
+                    const T* gp = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + pos;
+                    const T* gsafe = gp;                               // a legal address for masked rows
+                    const size_t wstep = (size_t)KL * P.Cgp, gstep = (size_t)KL * P.outV;
+                    const int ksteps = (P.M + KL - 1) / KL;
+                    // software pipeline: the loads of batch i+1 are in flight while the MFMAs of batch i run
+                    T a_nx[AB], b_nx[AB];
+                    auto load_batch = [&](int k0) {
 #pragma unroll
                         for (int k = 0; k < AB; ++k) {
-                            areg[k] = wu[a_off];
-                            wu += (size_t)KL * P.Cgp;
+                            a_nx[k] = wp[k * wstep];                   // rows past M are zero padding
+                            const bool ok = (k0 + k) * KL + q < P.M;
+                            const T* pb = ok ? gp + k * gstep : gsafe;
+                            b_nx[k] = *pb;
+                            if (!(ok && valid)) b_nx[k] = 0;
                         }
+                        wp += AB * wstep;
+                        gp += AB * gstep;
+                    };
+#ifndef RT_NOMFMA
+                    load_batch(0);
+                    for (int k0 = 0; k0 < ksteps; k0 += AB) {
+                        T a_cu[AB], b_cu[AB];
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) { a_cu[k] = a_nx[k]; b_cu[k] = b_nx[k]; }
+                        if (k0 + AB < ksteps) load_batch(k0 + AB);
                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) d = MM::mma(areg[k], breg[k0 + k], d);
+                        for (int k = 0; k < AB; ++k) d = MM::mma(a_cu[k], b_cu[k], d);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                } else {
-                    const T* gq = gq0;
-                    for (int m0 = 0; m0 < P.M; m0 += KL) {
-                        const T b = (valid && m0 + q < P.M) ? *gq : (T)0;
-                        d = MM::mma(wu[a_off], b, d);
-                        wu += (size_t)KL * P.Cgp;
-                        gq += (size_t)KL * P.outV;
-                    }
+#endif
                 }
+#ifdef RT_ONESLOT
+                for (int ts = 0; ts < 1; ++ts) {
+#else
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
+#endif
                     const int tap = tap_s[ts];
                     int kk[ND], kd[ND];
                     decode_tap<ND>(P, min(tap, P.kV - 1), kk);
@@ -871,13 +877,18 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                                 Cell* plane = sG + cl * P.hstride;
                                 const double gs = LdsCell<T>::pre(gv, scale);
 #pragma unroll
+#ifndef RT_NOFIX
                                 for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+#else
+                                for (int i = 0; i < NC; ++i) plane[lidx[i]] = (Cell)(cw[i] * gv);
+#endif
                                 if constexpr (COORD) {
                                     const T* ip = sIn + cl * P.hstride;
 #pragma unroll
                                     for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
                                 }
                             } else {
+#ifndef RT_NOFAR
                                 T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
 #pragma unroll
                                 for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
@@ -886,8 +897,15 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 #pragma unroll
                                     for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
                                 }
+#else
+                                for (int i = 0; i < NC; ++i) v[i] = 0;
+#endif
                             }
+#ifdef RT_NOCOORDMATH
+                            if constexpr (false) {
+#else
                             if constexpr (COORD) {
+#endif
                                 if constexpr (ND == 3) {
                                     const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh,
                                             fw = t.f[2], gw = (T)1 - fw;
@@ -932,7 +950,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                             T* gp = goff_dg + (size_t)tap * ND * P.outV + pos;
 #pragma unroll
                             for (int a = 0; a < ND; ++a) {
-                                if (first_chunk) gp[(size_t)a * P.outV] = ga[a];
+                                if (csplit > 1) { if (ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, ga[a]); }
+                                else if (first_chunk) gp[(size_t)a * P.outV] = ga[a];
                                 else gp[(size_t)a * P.outV] += ga[a];
                             }
                         }
