@@ -61,7 +61,15 @@ template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t i
     fwd_weight_pad<T>(M, Cg, MT, mchunks, Mp, Cgp);
     const size_t fwd = (size_t)G * kV * Mp * Cgp * sizeof(T);
     const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
-    const size_t bww = align256((size_t)N * C_in * inV * sizeof(T)) + align256((size_t)N * C_out * outV * sizeof(T));
+    // backward_weight: two channels-last copies + one partial weight per position split (at most 256 splits,
+    // and never more than about 4096 workgroups: see bww_plan)
+    const int TNq = Mma<T>::TN;
+    const long long tiles_lb = (long long)kV * ((C_in + TNq - 1) / TNq);           // lower bound of kV * nct * mchunks
+    long long split_ub = (4096 + tiles_lb - 1) / tiles_lb;
+    if (split_ub > 256) split_ub = 256;
+    if (split_ub < 1) split_ub = 1;
+    const size_t bww = align256((size_t)N * C_in * inV * sizeof(T)) + align256((size_t)N * C_out * outV * sizeof(T)) +
+                       align256((size_t)split_ub * kV * C_out * Cg * sizeof(T));
     size_t need = fwd > bwd ? fwd : bwd;
     return need > bww ? need : bww;
 }
@@ -353,14 +361,57 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     return check_launch("add_from_channels_last_kernel");
 }
 
+// Plan of backward_weight: channel tiles, m chunks and the number of position splits.
+template <typename T>
+void bww_plan(const Params& Pin, int& MT, int& mchunks, int& nct, int& nsplit) {
+    const int TN = Mma<T>::TN;
+    const int mtiles = (Pin.M + TN - 1) / TN;
+    MT = mtiles > 2 ? 4 : mtiles;
+    mchunks = (mtiles + MT - 1) / MT;
+    // channel tiles: one per TN channels of every (convolution group x deformable group) segment
+    nct = 0;
+    for (int gg = 0; gg < Pin.G; ++gg) {
+        const int cg0 = gg * Pin.Cg, cg1 = cg0 + Pin.Cg;
+        for (int dg = cg0 / Pin.cpg; dg <= (cg1 - 1) / Pin.cpg; ++dg) {
+            const int cb = cg0 > dg * Pin.cpg ? cg0 : dg * Pin.cpg;
+            const int ce = cg1 < (dg + 1) * Pin.cpg ? cg1 : (dg + 1) * Pin.cpg;
+            nct += (ce - cb + TN - 1) / TN;
+        }
+    }
+    // split the position reduction so that the grid holds a few thousand workgroups
+    const long long slabs = (long long)Pin.N * ((Pin.outV + TN - 1) / TN);
+    const long long other = (long long)Pin.kV * nct * mchunks;
+    long long split = (4096 + other - 1) / other;
+    const long long max_split = (slabs + WAVES - 1) / WAVES;
+    if (split > max_split) split = max_split;
+    if (split > 256) split = 256;
+    if (split < 1) split = 1;
+    nsplit = (int)split;
+}
+
 template <typename T, int ND, int MT>
-int launch_bwd_weight(const Params& P, const T* in_cl, const T* off, const T* gout_cl, T* gw, hipStream_t s) {
+int launch_bwd_weight(const Params& P, const T* in_cl, const T* off, const T* gout_cl, T* partial, hipStream_t s) {
+    const int TN = Mma<T>::TN;
+    const size_t lds = (size_t)WAVES * MT * TN * (TN + 1) * sizeof(T);
+    auto kern = backward_weight_kernel<T, ND, MT>;
+    if (lds > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
+        }
+    }
     const dim3 grid((unsigned)P.nsplit, (unsigned)P.kV, (unsigned)(P.nctiles * P.mchunks));
-    hipLaunchKernelGGL((backward_weight_kernel<T, ND, MT>), grid, dim3(WG), 0, s, P, in_cl, off, gout_cl, gw);
+    hipLaunchKernelGGL(kern, grid, dim3(WG), lds, s, P, in_cl, off, gout_cl, partial);
     return check_launch("backward_weight_kernel");
 }
 
-// Workspace of backward_weight: [ input channels-last | grad_output channels-last ]
+template <typename T> size_t bww_workspace(const Params& P, int nsplit) {
+    return align256((size_t)P.N * P.C_in * P.inV * sizeof(T)) + align256((size_t)P.N * P.C_out * P.outV * sizeof(T)) +
+           align256((size_t)nsplit * P.kV * P.C_out * P.Cg * sizeof(T));
+}
+
+// Workspace of backward_weight: [ input channels-last | grad_output channels-last | partial tiles per split ]
 template <typename T, int ND>
 int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout, T* gw, void* ws, size_t ws_bytes,
                     hipStream_t s) {
@@ -368,11 +419,15 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     if (int rc = validate(g, P)) return rc;
     if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     if ((long long)P.outV * P.C_out > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one output sample exceeds 2^31 elements");
+    int MT;
+    bww_plan<T>(P, MT, P.mchunks, P.nctiles, P.nsplit);
+    if ((long long)P.nctiles * P.mchunks > 65535) return fail(DCN_E_ARGUMENT, "too many channel tiles for one launch");
     const size_t ibytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
     const size_t obytes = align256((size_t)P.N * P.C_out * P.outV * sizeof(T));
-    if (!ws || ws_bytes < ibytes + obytes) return fail(DCN_E_WORKSPACE, "workspace too small");
+    if (!ws || ws_bytes < bww_workspace<T>(P, P.nsplit)) return fail(DCN_E_WORKSPACE, "workspace too small");
     T* in_cl = static_cast<T*>(ws);
     T* gout_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + ibytes);
+    T* partial = reinterpret_cast<T*>(static_cast<char*>(ws) + ibytes + obytes);
     const dim3 tblock(32, 8);
     hipLaunchKernelGGL(to_channels_last_kernel<T>, dim3((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N),
                        tblock, 0, s, in, in_cl, P.C_in, P.inV);
@@ -380,35 +435,17 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     hipLaunchKernelGGL(to_channels_last_kernel<T>, dim3((P.outV + 31) / 32, (unsigned)(P.C_out + 31) / 32, (unsigned)P.N),
                        tblock, 0, s, gout, gout_cl, P.C_out, P.outV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
-    const int TN = Mma<T>::TN;
-    const int mtiles = (P.M + TN - 1) / TN;
-    const int MT = mtiles > 2 ? 4 : mtiles;
-    P.mchunks = (mtiles + MT - 1) / MT;
-    // channel tiles: one per TN channels of every (convolution group x deformable group) segment
-    int nct = 0;
-    for (int gg = 0; gg < P.G; ++gg) {
-        const int cg0 = gg * P.Cg, cg1 = cg0 + P.Cg;
-        for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
-            const int cb = cg0 > dg * P.cpg ? cg0 : dg * P.cpg;
-            const int ce = cg1 < (dg + 1) * P.cpg ? cg1 : (dg + 1) * P.cpg;
-            nct += (ce - cb + TN - 1) / TN;
-        }
-    }
-    P.nctiles = nct;
-    if ((long long)nct * P.mchunks > 65535) return fail(DCN_E_ARGUMENT, "too many channel tiles for one launch");
-    // split the position reduction so that the grid holds a few thousand workgroups
-    const long long slabs = (long long)P.N * ((P.outV + TN - 1) / TN);
-    const long long other = (long long)P.kV * nct * P.mchunks;
-    long long split = (4096 + other - 1) / other;
-    const long long max_split = (slabs + WAVES - 1) / WAVES;
-    if (split > max_split) split = max_split;
-    if (split < 1) split = 1;
-    P.nsplit = (int)split;
+    int rc;
     switch (MT) {
-        case 1: return launch_bwd_weight<T, ND, 1>(P, in_cl, off, gout_cl, gw, s);
-        case 2: return launch_bwd_weight<T, ND, 2>(P, in_cl, off, gout_cl, gw, s);
-        default: return launch_bwd_weight<T, ND, 4>(P, in_cl, off, gout_cl, gw, s);
+        case 1: rc = launch_bwd_weight<T, ND, 1>(P, in_cl, off, gout_cl, partial, s); break;
+        case 2: rc = launch_bwd_weight<T, ND, 2>(P, in_cl, off, gout_cl, partial, s); break;
+        default: rc = launch_bwd_weight<T, ND, 4>(P, in_cl, off, gout_cl, partial, s); break;
     }
+    if (rc) return rc;
+    const size_t rows_x_cg = (size_t)P.C_out * P.Cg, total = rows_x_cg * P.kV;
+    const unsigned rb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+    hipLaunchKernelGGL(reduce_weight_partials_kernel<T>, dim3(rb), dim3(256), 0, s, partial, gw, P.nsplit, P.kV, rows_x_cg);
+    return check_launch("reduce_weight_partials_kernel");
 }
 
 Geometry geo3(int batch, int input_c, int output_c, int input_l, int input_h, int input_w, int output_l,

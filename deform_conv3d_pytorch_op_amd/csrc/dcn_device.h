@@ -173,22 +173,34 @@ __device__ inline void tap_setup(const Params& P, const T offv[ND], const int ib
 // Interpolated value of one channel: lerp along w, then h, then l (reference order,
 // deform3d kernel.cu:48-56, deform2d_double kernel.cu:50-53).  `chan` points at the channel's
 // first voxel; `voff` are the corner offsets (possibly biased by the caller, see kernels).
+// Split into the loads and the arithmetic so that callers can keep the loads of the next step in
+// flight while the current one is interpolated.
 template <typename T, int ND>
-__device__ inline T sample(const T* __restrict__ chan, const unsigned* voff, const T* f) {
+__device__ inline void load_corners(const T* __restrict__ chan, const unsigned* voff, T c[1 << ND]) {
+#pragma unroll
+    for (int i = 0; i < (1 << ND); ++i) c[i] = chan[voff[i]];
+}
+
+template <typename T, int ND>
+__device__ inline T interp(const T c[1 << ND], const T* f) {
     if constexpr (ND == 3) {
-        const T c000 = chan[voff[0]], c001 = chan[voff[1]], c010 = chan[voff[2]], c011 = chan[voff[3]];
-        const T c100 = chan[voff[4]], c101 = chan[voff[5]], c110 = chan[voff[6]], c111 = chan[voff[7]];
         const T fw = f[2], gw = (T)1 - fw, fh = f[1], gh = (T)1 - fh, fl = f[0], gl = (T)1 - fl;
-        const T c00 = c000 * gw + c001 * fw, c01 = c010 * gw + c011 * fw;
-        const T c10 = c100 * gw + c101 * fw, c11 = c110 * gw + c111 * fw;
+        const T c00 = c[0] * gw + c[1] * fw, c01 = c[2] * gw + c[3] * fw;
+        const T c10 = c[4] * gw + c[5] * fw, c11 = c[6] * gw + c[7] * fw;
         const T c0 = c00 * gh + c01 * fh, c1 = c10 * gh + c11 * fh;
         return c0 * gl + c1 * fl;
     } else {
-        const T c00 = chan[voff[0]], c01 = chan[voff[1]], c10 = chan[voff[2]], c11 = chan[voff[3]];
         const T fw = f[1], gw = (T)1 - fw, fh = f[0], gh = (T)1 - fh;
-        const T c0 = c00 * gw + c01 * fw, c1 = c10 * gw + c11 * fw;
+        const T c0 = c[0] * gw + c[1] * fw, c1 = c[2] * gw + c[3] * fw;
         return c0 * gh + c1 * fh;
     }
+}
+
+template <typename T, int ND>
+__device__ inline T sample(const T* __restrict__ chan, const unsigned* voff, const T* f) {
+    T c[1 << ND];
+    load_corners<T, ND>(chan, voff, c);
+    return interp<T, ND>(c, f);
 }
 
 __device__ inline void atomic_add(float* p, float v) { unsafeAtomicAdd(p, v); }

@@ -986,17 +986,19 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 // to the channel lanes through a wavefront-private LDS record.
 // A workgroup keeps one (tap, channel tile, m chunk) for its whole life; its wavefronts stride
 // over position slabs independently (no workgroup barriers), so the [MT*TN x TN] accumulator
-// stays in registers; partial sums of different wavefronts meet in grad_weight through
-// hardware float atomics.
-// grid.x = nsplit, grid.y = kV, grid.z = nctiles * mchunks.
+// stays in registers; each workgroup writes one partial tile per split and a small second kernel
+// sums the splits into grad_weight (deterministic, no atomics).
+// grid.x = nsplit, grid.y = kV, grid.z = nctiles * mchunks; dynamic LDS = WAVES * MT*TN * (TN+1) * sizeof(T).
 template <typename T, int ND, int MT>
 __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* __restrict__ in_cl,
                                                              const T* __restrict__ off,
-                                                             const T* __restrict__ gout_cl, T* __restrict__ gw) {
+                                                             const T* __restrict__ gout_cl, T* __restrict__ partial) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
     __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // corner voxel index * C_in, 0 when the sample is dead
     __shared__ __align__(16) T sF[WAVES][TN][4];             // f[ND]; [3] = 1 when the sample is live
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sAcc = reinterpret_cast<T*>(smem_raw);                // [WAVES][MT*TN][TN + 1]: the wavefronts' partial tiles
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
 
@@ -1072,39 +1074,86 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 
         const T* in_n = in_cl + (size_t)n * P.inV * P.C_in + cj;
         const T* go_n = gout_cl + (size_t)n * P.outV * P.C_out;
-#pragma unroll 4
-        for (int ks = 0; ks < TN / KL; ++ks) {
-            const int pp = ks * KL + q;                        // position of the slab this lane group works on
+        // reduction over the slab's positions, software pipelined: while step ks is interpolated and
+        // multiplied, the geometry record, the corner values and the grad_output rows of step ks + 1
+        // are already in flight
+        constexpr int NK = TN / KL;
+        T cn[NC], an[MT], fn[ND];                   // "next" step
+        bool lvn, okn;
+        auto fetch = [&](int ks) {
+            const int pp = ks * KL + q;             // position of the slab this lane group works on
             unsigned ix[NC];
 #pragma unroll
             for (int i = 0; i < NC; ++i) ix[i] = sIdx[wave][pp][i];
-            T f[ND];
 #pragma unroll
-            for (int a = 0; a < ND; ++a) f[a] = sF[wave][pp][a];
-            const bool lv = sF[wave][pp][3] != (T)0;
-            const T v = sample<T, ND>(in_n, ix, f);
-            const T b = (lv && chan_ok) ? v : (T)0;                                    // B[k = position][col = channel j]
+            for (int a_ = 0; a_ < ND; ++a_) fn[a_] = sF[wave][pp][a_];
+            lvn = sF[wave][pp][3] != (T)0;
             const unsigned pg = min(p0 + (unsigned)pp, P.outV - 1);
-            const bool p_ok = p0 + (unsigned)pp < P.outV;
+            okn = p0 + (unsigned)pp < P.outV;
             const T* grow = go_n + (size_t)pg * P.C_out;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const T a = grow[mrow[mt]];                                             // A[row = m][k = position]
-                acc[mt] = MM::mma((p_ok && m_ok[mt]) ? a : (T)0, b, acc[mt]);
-            }
+            for (int mt = 0; mt < MT; ++mt) an[mt] = grow[mrow[mt]];      // A[row = m][k = position]; legal for every lane
+            load_corners<T, ND>(in_n, ix, cn);                           // dead samples read voxel 0
+        };
+        fetch(0);
+#ifdef RT_BW_NOKLOOP
+        for (int ks = 0; ks < 1; ++ks) {
+#else
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks) {
+#endif
+            T cc[NC], ac[MT], fc[ND];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) cc[i] = cn[i];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) ac[mt] = an[mt];
+#pragma unroll
+            for (int a_ = 0; a_ < ND; ++a_) fc[a_] = fn[a_];
+            const bool lvc = lvn, okc = okn;
+            if (ks + 1 < NK) fetch(ks + 1);
+            __builtin_amdgcn_sched_barrier(0);      // next step's loads are issued before this step's arithmetic
+            const T v = interp<T, ND>(cc, fc);
+            const T b = (lvc && chan_ok) ? v : (T)0;                                   // B[k = position][col = channel j]
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma((okc && m_ok[mt]) ? ac[mt] : (T)0, b, acc[mt]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
-    const int c = c0 + j;
-    if (c >= ce) return;
+    // The four wavefronts' tiles are summed through LDS and the workgroup writes ONE partial tile
+    // to its own slot of the workspace: partial[split][tap][g*M + m][c_local].  (Float atomics
+    // straight into grad_weight cost 1.6 ms at 64x64x27 weights: a few hundred writers per address.)
+    constexpr int LDA = TN + 1;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int r = 0; r < MM::NACC; ++r) {
-            const int m = m_base + mt * TN + MM::row(r, q);
-            if (m < P.M)
-                atomic_add(gw + (((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap, acc[mt][r]);
+        for (int r = 0; r < MM::NACC; ++r)
+            sAcc[((size_t)wave * MT * TN + mt * TN + MM::row(r, q)) * LDA + j] = acc[mt][r];
+    __syncthreads();
+    T* pt = partial + ((size_t)blockIdx.x * P.kV + tap) * P.C_out * P.Cg;
+    for (int e = threadIdx.x; e < MT * TN * TN; e += WG) {
+        const int mr = e / TN, cc = e % TN;
+        const int m = m_base + mr, c = c0 + cc;
+        if (m < P.M && c < ce) {
+            T sum = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) sum += sAcc[((size_t)w * MT * TN + mr) * LDA + cc];
+            pt[((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)] = sum;
         }
+    }
+}
+
+// grad_weight[g*M+m][cl][tap] += sum over splits of partial[split][tap][g*M+m][cl]
+template <typename T>
+__global__ void reduce_weight_partials_kernel(const T* __restrict__ partial, T* __restrict__ gw, int nsplit, int kV,
+                                              size_t rows_x_cg /* C_out * Cg */) {
+    const size_t total = (size_t)kV * rows_x_cg;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t tap = i / rows_x_cg, rc = i % rows_x_cg;         // rc = (g*M + m) * Cg + cl
+        T sum = 0;
+        for (int s = 0; s < nsplit; ++s) sum += partial[((size_t)s * kV + tap) * rows_x_cg + rc];
+        gw[rc * kV + tap] += sum;
+    }
 }
 
 }  // namespace dcn
