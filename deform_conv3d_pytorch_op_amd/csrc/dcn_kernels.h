@@ -822,7 +822,6 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                         wp += AB * wstep;
                         gp += AB * gstep;
                     };
-#ifndef RT_NOMFMA
                     load_batch(0);
                     for (int k0 = 0; k0 < ksteps; k0 += AB) {
                         T a_cu[AB], b_cu[AB];
@@ -834,14 +833,9 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                         for (int k = 0; k < AB; ++k) d = MM::mma(a_cu[k], b_cu[k], d);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-#endif
                 }
-#ifdef RT_ONESLOT
-                for (int ts = 0; ts < 1; ++ts) {
-#else
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
-#endif
                     const int tap = tap_s[ts];
                     int kk[ND], kd[ND];
                     decode_tap<ND>(P, min(tap, P.kV - 1), kk);
@@ -877,18 +871,13 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                                 Cell* plane = sG + cl * P.hstride;
                                 const double gs = LdsCell<T>::pre(gv, scale);
 #pragma unroll
-#ifndef RT_NOFIX
                                 for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
-#else
-                                for (int i = 0; i < NC; ++i) plane[lidx[i]] = (Cell)(cw[i] * gv);
-#endif
                                 if constexpr (COORD) {
                                     const T* ip = sIn + cl * P.hstride;
 #pragma unroll
                                     for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
                                 }
                             } else {
-#ifndef RT_NOFAR
                                 T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
 #pragma unroll
                                 for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
@@ -897,15 +886,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 #pragma unroll
                                     for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
                                 }
-#else
-                                for (int i = 0; i < NC; ++i) v[i] = 0;
-#endif
                             }
-#ifdef RT_NOCOORDMATH
-                            if constexpr (false) {
-#else
                             if constexpr (COORD) {
-#endif
                                 if constexpr (ND == 3) {
                                     const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh,
                                             fw = t.f[2], gw = (T)1 - fw;
@@ -1096,12 +1078,8 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
             load_corners<T, ND>(in_n, ix, cn);                           // dead samples read voxel 0
         };
         fetch(0);
-#ifdef RT_BW_NOKLOOP
-        for (int ks = 0; ks < 1; ++ks) {
-#else
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks) {
-#endif
             T cc[NC], ac[MT], fc[ND];
 #pragma unroll
             for (int i = 0; i < NC; ++i) cc[i] = cn[i];
