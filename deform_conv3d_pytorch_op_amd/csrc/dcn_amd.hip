@@ -132,7 +132,8 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 // Returns false when the geometry does not suit (halo too large for the staging table or LDS).
 // Tuning knobs (environment, read once per process):
 //   DCN_HALO_MARGIN        voxels of halo beyond the integer tap span on each side (default 2)
-//   DCN_LDS_BUDGET_KB      LDS per workgroup of the forward halo kernel (default 72: two workgroups per CU)
+//   DCN_LDS_BUDGET_KB      LDS per 512-thread workgroup of the forward halo kernel (default 72: two per CU)
+//   DCN_FORWARD_WG=512     never use the 1024-thread forward variant; =1024 use it whenever its halo fits
 //   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
@@ -158,6 +159,13 @@ static int cu_count() {
     }();
     return v;
 }
+static int wide_forward() {      // 0 never, 1 when it pays, 2 whenever the halo fits
+    static const int v = [] {
+        const char* e = getenv("DCN_FORWARD_WG");
+        return !e ? 1 : atoi(e) == 512 ? 0 : atoi(e) == 1024 ? 2 : 1;
+    }();
+    return v;
+}
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
     return v != 0;
@@ -175,8 +183,8 @@ int halo_margin() {
 }
 
 template <typename T, int ND>
-bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T)) {
-    const int npos = WAVESH * Mma<T>::TN;       // positions per workgroup: 256 (float) or 128 (double)
+bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH) {
+    const int npos = waves * Mma<T>::TN;        // positions per workgroup, one column tile per wavefront
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
     else         { td[2] = 16; td[1] = npos / 16; }
@@ -211,7 +219,7 @@ bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_by
 }
 
 template <typename K, typename... Args>
-int launch_halo(K kern, const char* name, dim3 grid, size_t lds, hipStream_t s, Args... args) {
+int launch_halo(K kern, const char* name, dim3 grid, int threads, size_t lds, hipStream_t s, Args... args) {
     if (lds > 64 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)lds) != hipSuccess) {
@@ -219,7 +227,7 @@ int launch_halo(K kern, const char* name, dim3 grid, size_t lds, hipStream_t s, 
             return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
         }
     }
-    hipLaunchKernelGGL(kern, grid, dim3(WGH), lds, s, args...);
+    hipLaunchKernelGGL(kern, grid, dim3(threads), lds, s, args...);
     return check_launch(name);
 }
 
@@ -235,17 +243,29 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     T* wt = static_cast<T*>(ws);
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     const int TN = Mma<T>::TN;
-    // two workgroups per CU when that still leaves 8 channels per LDS pass, else one large one
+    // Few accumulators (MT <= 2): one 1024-thread workgroup per CU with the whole LDS, if its larger
+    // halo fits and leaves 8 channels per pass.  Otherwise 512 threads: two workgroups per CU when
+    // that still leaves 8 channels per LDS pass, else one large one.
+    if (MT <= 2 && wide_forward()) {
+        Params Pw = P;
+        if (plan_halo<T, ND>(Pw, 144 * 1024, 1 << 30, sizeof(T), 16) &&
+            (wide_forward() == 2 || (Pw.cchunk >= 8 && (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks >= cu_count()))) {
+            const size_t lds = (size_t)Pw.cchunk * Pw.hstride * sizeof(T) + (size_t)Pw.hvol * 4;
+            const dim3 grid((unsigned)Pw.N * Pw.tiles, (unsigned)Pw.G * Pw.mchunks);
+            if (MT == 1) return launch_halo(forward_halo_kernel<T, ND, 1, 16>, "forward_halo_kernel", grid, 1024, lds, s, Pw, in, off, wt, bias, out);
+            return launch_halo(forward_halo_kernel<T, ND, 2, 16>, "forward_halo_kernel", grid, 1024, lds, s, Pw, in, off, wt, bias, out);
+        }
+    }
     bool tiled = plan_halo<T, ND>(P, LDS_BUDGET);
     if ((!tiled || P.cchunk < 8) && LDS_BUDGET < 144 * 1024) tiled = plan_halo<T, ND>(P, 144 * 1024) || tiled;
     if (tiled) {
         const size_t lds = (size_t)P.cchunk * P.hstride * sizeof(T) + (size_t)P.hvol * 4;
         const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
         switch (MT) {
-            case 1: return launch_halo(forward_halo_kernel<T, ND, 1>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
-            case 2: return launch_halo(forward_halo_kernel<T, ND, 2>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
-            case 4: return launch_halo(forward_halo_kernel<T, ND, 4>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
-            default: return launch_halo(forward_halo_kernel<T, ND, 8>, "forward_halo_kernel", grid, lds, s, P, in, off, wt, bias, out);
+            case 1: return launch_halo(forward_halo_kernel<T, ND, 1, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
+            case 2: return launch_halo(forward_halo_kernel<T, ND, 2, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
+            case 4: return launch_halo(forward_halo_kernel<T, ND, 4, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
+            default: return launch_halo(forward_halo_kernel<T, ND, 8, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
         }
     }
     // geometry whose halo does not fit in LDS: gather straight from global memory
@@ -287,9 +307,9 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     // 1) one kernel: scatter privatised in LDS + coordinate gradient from an LDS input halo
     Params Ph = P;
     if (scatter_in_lds() && fused_coord() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T)) &&
-        (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4) {
+        (scatter_budget() - (size_t)Ph.hvol * 4 - (size_t)P.kV * ND * 4) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4) {
         Ph.cchunk = 4;
-        const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4;
+        const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
         hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
         if (int rc = check_launch("absmax_kernel")) return rc;
         // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
@@ -304,6 +324,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (rounds < best * 0.97) { best = rounds; csplit = cs; }
         }
         if (const char* e = getenv("DCN_CSPLIT")) csplit = atoi(e) > 0 ? atoi(e) : csplit;
+        if (csplit > nchunks) csplit = nchunks;
         if (csplit > 1) {
             const size_t nel = (size_t)P.N * P.DG * P.kV * ND * P.outV;
             const unsigned fb = (unsigned)((nel + 1023) / 1024 > 8192 ? 8192 : (nel + 1023) / 1024);
@@ -311,7 +332,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (int rc = check_launch("fill_zero_kernel")) return rc;
         }
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG, (unsigned)csplit);
-        return launch_halo(backward_input_halo_kernel<T, ND, 4, true>, "backward_input_halo_kernel", hgrid, lds, s, Ph,
+        return launch_halo(backward_input_halo_kernel<T, ND, 4, true>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
                            in, off, wt, gout, wmax, gin, goff);
     }
 
@@ -321,7 +342,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     Ph = P;
     bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
     if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
-        const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * 8);
+        const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4 - (size_t)P.kV * ND * 4) / ((size_t)Ph.hstride * 8);
         if (fit >= 8) Ph.cchunk = 8;
         else if (fit >= 4) Ph.cchunk = 4;
         else halo = false;
@@ -337,16 +358,16 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             default: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
         }
         if (int rc = check_launch("backward_data_kernel")) return rc;
-        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4;
+        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
         hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
         if (int rc = check_launch("absmax_kernel")) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)
-            return launch_halo(backward_input_halo_kernel<T, ND, 8, false>, "backward_input_halo_kernel", hgrid, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 8, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff);
         if (Ph.cchunk == 4)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, false>, "backward_input_halo_kernel", hgrid, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }

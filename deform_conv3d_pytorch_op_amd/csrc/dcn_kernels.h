@@ -112,8 +112,8 @@ __global__ __launch_bounds__(WG) void forward_kernel(Params P, const T* __restri
 }
 
 // ---------------------------------------------------------------------------------------------
-// Halo tiling.  A workgroup of WGH threads owns a compact block of output positions
-// (tdim[0] x tdim[1] x tdim[2], WAVESH * TN of them) and stages the input neighbourhood that the
+// Halo tiling.  A workgroup of WGH threads (1024 in the light forward variants) owns a compact
+// block of output positions (tdim[0] x tdim[1] x tdim[2], one TN-wide column tile per wavefront) and stages the input neighbourhood that the
 // block's samples can reach -- the "halo" -- in LDS, `cchunk` channels at a time, as channel
 // planes [channel][halo voxel].  Samples whose corners all fall inside the halo are interpolated
 // from LDS; the few that reach further (large offsets) fall back to global memory, so any offset
@@ -167,9 +167,9 @@ __device__ inline bool tile_position(const Params& P, const TileGeo<ND>& tg, int
 // Table of the halo: for every halo voxel its offset inside one channel of the input, or ~0u
 // where the halo sticks out of the volume.  Built once per workgroup into LDS (hvol entries) so
 // that staging, zeroing and flushing need no per-thread index math and no registers.
-template <int ND>
+template <int ND, int WGS = WGH>
 __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsigned* __restrict__ sTab) {
-    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGH) {
+    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGS) {
         int v = v0;
         bool inb = true;
         unsigned lin = 0;
@@ -189,14 +189,14 @@ __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsign
 
 // Stage `nch` channel planes of the halo.  Halo voxels outside the volume are never read by a
 // sample; they are staged from voxel 0 so that every load is unconditional.
-template <typename T>
+template <typename T, int WGS = WGH>
 __device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, int nch,
                                   const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
-    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGH * 4) {
+    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGS * 4) {
         unsigned g[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const int v = v0 + WGH * k;
+            const int v = v0 + WGS * k;
             const unsigned t = v < P.hvol ? sTab[v] : ~0u;
             g[k] = t == ~0u ? 0u : t;
         }
@@ -207,7 +207,7 @@ __device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, 
             for (int k = 0; k < 4; ++k) val[k] = ch[g[k]];              // four loads in flight
 #pragma unroll
             for (int k = 0; k < 4; ++k)
-                if (v0 + WGH * k < P.hvol) sIn[c * P.hstride + v0 + WGH * k] = val[k];
+                if (v0 + WGS * k < P.hvol) sIn[c * P.hstride + v0 + WGS * k] = val[k];
         }
     }
 }
@@ -239,10 +239,11 @@ __device__ inline bool halo_corners(const Params& P, const int hb[ND], const Tap
 
 // Forward with the input halo in LDS.  Same contraction and lane roles as forward_kernel; the
 // sampled value of lane (j, q) is the MFMA B operand B[k = q][col = j].
-// grid.x = N * tiles (3-D blocks of positions), grid.y = G * mchunks;
-// dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4.
-template <typename T, int ND, int MT>
-__global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __restrict__ in,
+// grid.x = N * tiles (3-D blocks of positions), grid.y = G * mchunks, NW wavefronts per workgroup
+// (16 when the accumulators are few enough for 128 registers: the larger block shares each staged
+// halo between twice the positions); dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4.
+template <typename T, int ND, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T* __restrict__ in,
                                                            const T* __restrict__ off, const T* __restrict__ Wt,
                                                            const T* __restrict__ bias, T* __restrict__ out) {
     using MM = Mma<T>;
@@ -262,7 +263,7 @@ __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __
     const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
-    halo_table<ND>(P, tg, sTab);                   // visible after the first barrier below
+    halo_table<ND, NW * 64>(P, tg, sTab);          // visible after the first barrier below
 
     typename MM::Acc acc[MT];
 #pragma unroll
@@ -276,7 +277,7 @@ __global__ __launch_bounds__(WGH) void forward_halo_kernel(Params P, const T* __
             const int nch = min(P.cchunk, ce - cc0);
             const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
             __syncthreads();                                               // readers of the previous chunk are done
-            halo_stage<T>(P, chan0, nch, sTab, sIn);
+            halo_stage<T, NW * 64>(P, chan0, nch, sTab, sIn);
             __syncthreads();
             const int nsteps = (nch + KL - 1) / KL;
             T onext[ND];
@@ -696,7 +697,7 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // atomics.  After all taps the planes are added to grad_input with one hardware float atomic per
 // touched halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that
 // reach past the halo use global atomics directly.
-// grid.x = N * tiles, grid.y = DG; dynamic LDS = CCH * hstride * 8 + hvol * 4 bytes.
+// grid.x = N * tiles, grid.y = DG; dynamic LDS = CCH * hstride * 8 + hvol * 4 + kV * ND * 4 bytes.
 // COORD = true additionally stages the same CCH input channels over the halo (float planes) and
 // computes grad_offset in the same pass over the grad-column values (col2im_offset of the
 // reference, deform3d kernel.cu:386-483 incl. the out-of-range branches :470-481, 2-D
@@ -721,6 +722,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
     T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * P.hstride);                        // [CCH][hstride] if COORD
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * P.hstride : 0));   // [hvol]
+    int* sKd = reinterpret_cast<int*>(sTab + P.hvol);                                   // [kV][ND]: tap * dilation per axis
     __shared__ float sRed[WAVESH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
@@ -739,6 +741,12 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
     halo_table<ND>(P, tg, sTab);                   // visible after the first barrier below
+    for (int tp = threadIdx.x; tp < P.kV; tp += WGH) {      // taps differ between lanes here: a table replaces the divisions
+        int kk[ND];
+        decode_tap<ND>(P, tp, kk);
+#pragma unroll
+        for (int a = 0; a < ND; ++a) sKd[tp * ND + a] = kk[a] * P.dil[slot<ND>(a)];
+    }
 
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
@@ -837,10 +845,9 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
                     const int tap = tap_s[ts];
-                    int kk[ND], kd[ND];
-                    decode_tap<ND>(P, min(tap, P.kV - 1), kk);
+                    int kd[ND];
 #pragma unroll
-                    for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+                    for (int a = 0; a < ND; ++a) kd[a] = sKd[min(tap, P.kV - 1) * ND + a];
                     TapGeo<T, ND> t;
                     tap_setup<T, ND>(P, ofs[ts], ib, kd, t);
                     const bool slot_ok = valid && tap < P.kV;

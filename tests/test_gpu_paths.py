@@ -5,6 +5,10 @@ settings, each in a process of its own (the knobs are read once per process):
   DCN_HALO_MARGIN=50   the halo never fits -> kernels that do not use LDS tiling at all
   DCN_SCATTER=global   grad-input through global atomics on the channels-last copy
   DCN_LDS_BUDGET_KB / DCN_SCATTER_BUDGET_KB small -> smallest channel chunks
+  DCN_FORWARD_WG=1024  the 1024-thread forward variant also where the grid would be too small for it
+  DCN_FORWARD_WG=512   ... and never
+  DCN_COORD=separate   grad_offset from the channels-last kernel, grad_input from the scatter-only kernel
+  DCN_CSPLIT=1 / 4     channel chunks of the fused backward kernel on one / four workgroups
 """
 import os
 import subprocess
@@ -20,6 +24,9 @@ SETTINGS = [
     {"DCN_HALO_MARGIN": "50"},
     {"DCN_SCATTER": "global"},
     {"DCN_LDS_BUDGET_KB": "16", "DCN_SCATTER_BUDGET_KB": "72"},
+    {"DCN_FORWARD_WG": "1024", "DCN_CSPLIT": "4"},
+    {"DCN_FORWARD_WG": "512", "DCN_CSPLIT": "1"},
+    {"DCN_COORD": "separate"},
 ]
 
 
