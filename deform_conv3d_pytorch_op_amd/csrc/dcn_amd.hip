@@ -332,7 +332,11 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (int rc = check_launch("fill_zero_kernel")) return rc;
         }
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG, (unsigned)csplit);
-        return launch_halo(backward_input_halo_kernel<T, ND, 4, true>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
+        // grad_output operand held in registers when its reduction steps fit (M <= 64 float, 128 double)
+        if ((P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32)
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true>, "backward_input_halo_kernel", hgrid, WGH, lds,
+                               s, Ph, in, off, wt, gout, wmax, gin, goff);
+        return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
                            in, off, wt, gout, wmax, gin, goff);
     }
 
@@ -364,10 +368,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)
-            return launch_halo(backward_input_halo_kernel<T, ND, 8, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff);
         if (Ph.cchunk == 4)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }

@@ -704,7 +704,9 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // deform2d_double kernel.cu:309-366): per (tap, position) the derivative of the interpolation
 // along each axis times gcol, summed over the chunk's channels, accumulated into grad_offset
 // chunk after chunk (the first chunk stores).  dynamic LDS then adds CCH * hstride * sizeof(T).
-template <typename T, int ND, int CCH, bool COORD>
+// BREG = true (host: at most NS * 8 reduction steps, i.e. M <= 64 for float) keeps this lane's
+// grad_output values -- the B operand, the same for every tap and channel chunk -- in registers.
+template <typename T, int ND, int CCH, bool COORD, bool BREG>
 __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
@@ -759,14 +761,31 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
-        const T* gq0 = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + pos;
+        // wave-uniform base (scalar registers) + 32-bit lane offset of the B operand grad_output[m][pos]
+        constexpr int AB = 8;                       // reduction steps per operand batch
+        const T* gbase = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV;
+        const unsigned b_off = (unsigned)q * P.outV + pos;
+        const size_t gstep = (size_t)KL * P.outV;
+        // Reduction step k of this lane.  Rows past M read row 0 of the same position instead (the
+        // weight rows they meet are zero padding) and lanes outside the volume read a clamped
+        // position (their columns are never used), so the load itself needs no mask; `masked`
+        // additionally zeroes both cases for the bound below.
+        auto load_b = [&](int k, bool masked) -> T {
+            const int row0 = k * KL;                // uniform
+            const bool ok = row0 + q < P.M;
+            const T* gb = gbase + (size_t)(row0 < P.M ? k : 0) * gstep;
+            const T b = gb[ok ? b_off : pos];
+            return (!masked || (ok && valid)) ? b : (T)0;
+        };
+        T b_reg[BREG ? NS * AB : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
-        {
-            const T* gq = gq0;
-            for (int m0 = 0; m0 < P.M; m0 += KL) {
-                if (valid && m0 + q < P.M) sabs += fabsf((float)*gq);
-                gq += (size_t)KL * P.outV;
-            }
+        if constexpr (BREG) {
+#pragma unroll
+            for (int k = 0; k < NS * AB; ++k) b_reg[k] = load_b(k, true);
+#pragma unroll
+            for (int k = 0; k < NS * AB; ++k) sabs += fabsf((float)b_reg[k]);
+        } else {
+            for (int k = 0; k * KL < P.M; ++k) sabs += fabsf((float)load_b(k, true));
         }
         // fixed-point exponent of this (workgroup, convolution group): terms are bounded by
         // 8 * max|W| * max_pos sum_m |grad_output|
@@ -794,85 +813,124 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
             if constexpr (COORD) halo_stage<T>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
 
-            for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
-                // offsets of this lane's tap slots travel while the MFMA pass runs
-                T ofs[NS][ND];
-                int tap_s[NS];
+            // Grad-column tile of a pass: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past
+            // the last one read zero padding (or rows that are ignored below).  The MFMAs of pass p+1
+            // are issued between the tap slots of pass p, a few per accumulator register walked, so
+            // the matrix pipe works behind the vector work of the scatter instead of before it.
+            // Operands arrive in batches of AB reduction steps, loaded one tap slot ahead of use.
+            constexpr int MPR = AB / RPS;                              // MFMAs per accumulator register walked
+            const size_t wstep = (size_t)KL * P.Cgp;
+            const size_t wpass = (size_t)TP * P.Mp * P.Cgp;            // weight slabs of one pass
+            const int ksteps = (P.M + KL - 1) / KL;
+            const T* wchunk = Wt + ((size_t)g * P.kV * P.Mp) * P.Cgp + (cc0 - g * P.Cg);      // uniform; lanes add a_off
+            // (k0 passes through an empty asm: what is derived from it is then computed where it is
+            // used instead of being hoisted out of the loops into hundreds of long-lived registers)
+            auto load_batch = [&](T* a_nx, T* b_nx, const T* wp, int k0) {      // rows past M are zero padding
+                asm volatile("" : "+s"(k0));
+#pragma unroll
+                for (int k = 0; k < AB; ++k) {
+                    a_nx[k] = (wp + (size_t)(k0 + k) * wstep)[a_off];
+                    if constexpr (!BREG) b_nx[k] = load_b(k0 + k, false);
+                }
+            };
+            // steps [k_begin, ksteps) of one pass in a software-pipelined loop of their own: the whole
+            // first pass, and what the tap slots cannot take when M is large
+            auto gemm_tail = [&](typename MM::Acc& dd, const T* wp, int k_begin) {
+                T a_nx[AB], b_nx[AB];
+                load_batch(a_nx, b_nx, wp, k_begin);
+                for (int k0 = k_begin; k0 < ksteps; k0 += AB) {
+                    T a_cu[AB], b_cu[AB];
+#pragma unroll
+                    for (int k = 0; k < AB; ++k) { a_cu[k] = a_nx[k]; b_cu[k] = b_nx[k]; }
+                    if (k0 + AB < ksteps) load_batch(a_nx, b_nx, wp, k0 + AB);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_cu[k], b_cu[k], dd);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            typename MM::Acc d_next = acc_zero<T>();
+            if constexpr (BREG) {                                      // first pass: nothing to hide behind
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
-                    tap_s[ts] = tap0 + MM::row(ts * RPS, q) / CCH;
-                    const int tl = min(tap_s[ts], P.kV - 1);
-                    load_offsets<T, ND>(P, off_dg + (size_t)tl * ND * P.outV, pos, ofs[ts]);
-                }
-                // grad-column tile: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past the
-                // last one read zero padding (or rows that are ignored below)
-                typename MM::Acc d = acc_zero<T>();
-                // operands in batches of AB reduction steps: all loads of a batch are issued before its
-                // MFMAs need them; a rolled loop with two running pointers keeps the address state small
-                {
-                    constexpr int AB = 8;
-                    const T* wp = Wt + (((size_t)g * P.kV + tap0) * P.Mp) * P.Cgp + (cc0 - g * P.Cg) + a_off;
-                    const T* gp = gout + ((size_t)n * P.C_out + (size_t)g * P.M + q) * P.outV + pos;
-                    const T* gsafe = gp;                               // a legal address for masked rows
-                    const size_t wstep = (size_t)KL * P.Cgp, gstep = (size_t)KL * P.outV;
-                    const int ksteps = (P.M + KL - 1) / KL;
-                    // software pipeline: the loads of batch i+1 are in flight while the MFMAs of batch i run
-                    T a_nx[AB], b_nx[AB];
-                    auto load_batch = [&](int k0) {
+                    if (ts * AB < ksteps) {
+                        T a_cu[AB];
+                        load_batch(a_cu, nullptr, wchunk, ts * AB);
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) {
-                            a_nx[k] = wp[k * wstep];                   // rows past M are zero padding
-                            const bool ok = (k0 + k) * KL + q < P.M;
-                            const T* pb = ok ? gp + k * gstep : gsafe;
-                            b_nx[k] = *pb;
-                            if (!(ok && valid)) b_nx[k] = 0;
-                        }
-                        wp += AB * wstep;
-                        gp += AB * gstep;
-                    };
-                    load_batch(0);
-                    for (int k0 = 0; k0 < ksteps; k0 += AB) {
-                        T a_cu[AB], b_cu[AB];
-#pragma unroll
-                        for (int k = 0; k < AB; ++k) { a_cu[k] = a_nx[k]; b_cu[k] = b_nx[k]; }
-                        if (k0 + AB < ksteps) load_batch(k0 + AB);
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int k = 0; k < AB; ++k) d = MM::mma(a_cu[k], b_cu[k], d);
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int k = 0; k < AB; ++k) d_next = MM::mma(a_cu[k], b_reg[ts * AB + k], d_next);
                     }
                 }
+            } else {
+                gemm_tail(d_next, wchunk, 0);
+            }
+            T o_nx[ND];                                                // offsets of the next tap slot
+            auto load_slot_offsets = [&](int tap_u, int ts) {         // tap_u: uniform tap of lane group 0 in slot ts
+                const int tu = min(tap_u, P.kV - 1);
+                const int dq = MM::row(ts * RPS, q) / CCH - MM::row(ts * RPS, 0) / CCH;
+                const unsigned lo = (tu + dq < P.kV ? (unsigned)dq * ND * P.outV : 0u) + pos;
+                const T* ob = off_dg + (size_t)tu * ND * P.outV;
+#pragma unroll
+                for (int a = 0; a < ND; ++a) o_nx[a] = (ob + (size_t)a * P.outV)[lo];
+            };
+            load_slot_offsets(MM::row(0, 0) / CCH, 0);
+
+            for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
+                const typename MM::Acc d = d_next;
+                d_next = acc_zero<T>();
+                const bool more = tap0 + TP < P.kV;                    // a pass follows: its MFMAs ride along
+                int kz = 0;                                            // an opaque zero, for the same reason
+                asm volatile("" : "+s"(kz));
+                const T* wnext = wchunk + (size_t)(tap0 / TP + 1) * wpass;
+                if constexpr (!BREG) { if (more && ksteps > NS * AB) gemm_tail(d_next, wnext, NS * AB); }
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
-                    const int tap = tap_s[ts];
+                    const int tap = tap0 + MM::row(ts * RPS, q) / CCH;
+                    T a_cu[AB], b_cu[AB], ofs[ND];
+#pragma unroll
+                    for (int a = 0; a < ND; ++a) ofs[a] = o_nx[a];
+                    const bool do_mma = more && ts * AB < ksteps;      // uniform
+                    // this slot's MFMA operands arrive while its geometry is set up; the offsets of the
+                    // next tap slot travel while this one is worked on
+                    if (do_mma) load_batch(a_cu, b_cu, wnext, ts * AB);
+                    if (ts + 1 < NS) load_slot_offsets(tap0 + MM::row((ts + 1) * RPS, 0) / CCH, ts + 1);
+                    else load_slot_offsets(tap0 + TP + MM::row(0, 0) / CCH, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+
                     int kd[ND];
 #pragma unroll
                     for (int a = 0; a < ND; ++a) kd[a] = sKd[min(tap, P.kV - 1) * ND + a];
                     TapGeo<T, ND> t;
-                    tap_setup<T, ND>(P, ofs[ts], ib, kd, t);
+                    tap_setup<T, ND>(P, ofs, ib, kd, t);
                     const bool slot_ok = valid && tap < P.kV;
                     const bool live = slot_ok && t.inside;
                     T ga[ND];
 #pragma unroll
                     for (int a = 0; a < ND; ++a) ga[a] = 0;
-                    if (live) {
-                        unsigned lidx[NC];
-                        const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
-                        T cw[NC];
-                        if constexpr (ND == 3) {   // multiplied in the reference's order (w_l * w_h * w_w)
-                            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
-                            cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
-                            cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
-                        } else {
-                            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                            cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
-                        }
+                    // corner cells and weights, computed by every lane (dead lanes never use them)
+                    unsigned lidx[NC];
+                    const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+                    T cw[NC];
+                    if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
+                        const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                        cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                        cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+                    } else {
+                        const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                        cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                    }
+                    // out-of-range samples of the 3-D operator: +-|gcol| per axis; h and w are compared
+                    // with the LENGTH extent
+                    const bool oor = COORD && ND == 3 && slot_ok && !t.inside;
+                    T sg[ND];
 #pragma unroll
-                        for (int rr = 0; rr < RPS; ++rr) {
-                            const int r = ts * RPS + rr;
-                            const int cl = MM::row(r, q) % CCH;
-                            if (cl >= nch) continue;
-                            const T gv = d[r];
+                    for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= (T)P.in[0]) ? (T)1 : (T)0);
+#pragma unroll
+                    for (int rr = 0; rr < RPS; ++rr) {
+                        const int r = ts * RPS + rr;
+                        const int cl = MM::row(r, q) % CCH;
+                        const T gv = d[r];
+                        if (cl >= nch) {
+                        } else if (live) {
                             T v[NC];
                             if (in_halo) {
                                 Cell* plane = sG + cl * P.hstride;
@@ -885,11 +943,12 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                                     for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
                                 }
                             } else {
-                                T* gc = gin + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
+                                const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
+                                T* gc = gin + chan;
 #pragma unroll
                                 for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
                                 if constexpr (COORD) {
-                                    const T* ic = in + ((size_t)n * P.C_in + cc0 + cl) * P.inV;
+                                    const T* ic = in + chan;
 #pragma unroll
                                     for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
                                 }
@@ -910,20 +969,16 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                                     ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
                                 }
                             }
-                        }
-                    } else if (COORD && ND == 3 && slot_ok) {
-                        // out-of-range sample: +-|gcol| per axis; h and w are compared with the LENGTH extent
-                        const T len = (T)P.in[0];
-                        T sg[ND];
-#pragma unroll
-                        for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= len) ? (T)1 : (T)0);
-#pragma unroll
-                        for (int rr = 0; rr < RPS; ++rr) {
-                            const int r = ts * RPS + rr;
-                            if (MM::row(r, q) % CCH >= nch) continue;
-                            const T av = d[r] > 0 ? d[r] : -d[r];
+                        } else if (oor) {
+                            const T av = gv > 0 ? gv : -gv;
 #pragma unroll
                             for (int a = 0; a < ND; ++a) ga[a] += sg[a] * av;
+                        }
+                        // the next pass's MFMAs of this step, in uniform control flow
+                        if (do_mma) {
+#pragma unroll
+                            for (int k = 0; k < MPR; ++k)
+                                d_next = MM::mma(a_cu[rr * MPR + k], BREG ? b_reg[ts * AB + rr * MPR + k] : b_cu[rr * MPR + k], d_next);
                         }
                     }
                     if constexpr (COORD) {
