@@ -280,6 +280,15 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     return check_launch("forward_kernel");
 }
 
+template <typename T>
+int absmax(const T* w, size_t n, float* out, hipStream_t s) {
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(1), dim3(64), 0, s, out, (size_t)1);
+    if (int rc = check_launch("fill_zero_kernel")) return rc;
+    const unsigned blocks = (unsigned)((n + 1023) / 1024 > 128 ? 128 : (n + 1023) / 1024);
+    hipLaunchKernelGGL(absmax_kernel<T>, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, n, out);
+    return check_launch("absmax_kernel");
+}
+
 template <typename T, int ND>
 int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* off, const T* gout, T* gin,
                           T* goff, void* ws, size_t ws_bytes, hipStream_t s) {
@@ -310,8 +319,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         (scatter_budget() - (size_t)Ph.hvol * 4 - (size_t)P.kV * ND * 4) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4) {
         Ph.cchunk = 4;
         const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
-        hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
-        if (int rc = check_launch("absmax_kernel")) return rc;
+        if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
         // wastes least of the last round (one workgroup per CU at this LDS size)
         const int nchunks = ((P.cpg < P.Cg ? P.cpg : P.Cg) + 3) / 4;
@@ -363,8 +371,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         }
         if (int rc = check_launch("backward_data_kernel")) return rc;
         const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
-        hipLaunchKernelGGL(absmax_kernel<T>, dim3(1), dim3(1024), 0, s, w, (size_t)P.C_out * P.Cg * P.kV, wmax);
-        if (int rc = check_launch("absmax_kernel")) return rc;
+        if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)

@@ -668,19 +668,22 @@ template <> struct LdsCell<double> {
     __device__ static inline double value(type c, double) { return c; }
 };
 
-// max |w| over a small tensor, one workgroup (used for the fixed-point exponent)
+// max |w| over a small tensor (used for the fixed-point exponent).  Each workgroup reduces a
+// strided share and joins the result with an integer atomic max: non-negative floats order like
+// their bit patterns.  `out` must hold 0 beforehand.
 template <typename T>
 __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restrict__ out) {
-    __shared__ float red[1024];
+    __shared__ float red[256];
     float m = 0.f;
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf((float)w[i]));
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        m = fmaxf(m, fabsf((float)w[i]));
     red[threadIdx.x] = m;
     __syncthreads();
     for (int sft = blockDim.x / 2; sft > 0; sft >>= 1) {
         if ((int)threadIdx.x < sft) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + sft]);
         __syncthreads();
     }
-    if (threadIdx.x == 0) out[0] = red[0];
+    if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned*>(out), __float_as_uint(red[0]));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -933,15 +936,17 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                         } else if (live) {
                             T v[NC];
                             if (in_halo) {
-                                Cell* plane = sG + cl * P.hstride;
-                                const double gs = LdsCell<T>::pre(gv, scale);
-#pragma unroll
-                                for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+                                // the reads go first: LDS operations complete in order, so the interpolation
+                                // gradient below waits for them only, not for the adds issued after them
                                 if constexpr (COORD) {
                                     const T* ip = sIn + cl * P.hstride;
 #pragma unroll
                                     for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
                                 }
+                                Cell* plane = sG + cl * P.hstride;
+                                const double gs = LdsCell<T>::pre(gv, scale);
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
                             } else {
                                 const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
                                 T* gc = gin + chan;
