@@ -866,14 +866,18 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
             } else {
                 gemm_tail(d_next, wchunk, 0);
             }
-            T o_nx[ND];                                                // offsets of the next tap slot
+            T o_nx[ND];                                                // offsets and tap * dilation of the next tap slot
+            int kd_nx[ND];
             auto load_slot_offsets = [&](int tap_u, int ts) {         // tap_u: uniform tap of lane group 0 in slot ts
                 const int tu = min(tap_u, P.kV - 1);
                 const int dq = MM::row(ts * RPS, q) / CCH - MM::row(ts * RPS, 0) / CCH;
-                const unsigned lo = (tu + dq < P.kV ? (unsigned)dq * ND * P.outV : 0u) + pos;
+                const int dqc = tu + dq < P.kV ? dq : 0;
+                const unsigned lo = (unsigned)dqc * ND * P.outV + pos;
                 const T* ob = off_dg + (size_t)tu * ND * P.outV;
 #pragma unroll
                 for (int a = 0; a < ND; ++a) o_nx[a] = (ob + (size_t)a * P.outV)[lo];
+#pragma unroll
+                for (int a = 0; a < ND; ++a) kd_nx[a] = sKd[(tu + dqc) * ND + a];
             };
             load_slot_offsets(MM::row(0, 0) / CCH, 0);
 
@@ -889,8 +893,9 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                 for (int ts = 0; ts < NS; ++ts) {
                     const int tap = tap0 + MM::row(ts * RPS, q) / CCH;
                     T a_cu[AB], b_cu[AB], ofs[ND];
+                    int kd[ND];
 #pragma unroll
-                    for (int a = 0; a < ND; ++a) ofs[a] = o_nx[a];
+                    for (int a = 0; a < ND; ++a) { ofs[a] = o_nx[a]; kd[a] = kd_nx[a]; }
                     const bool do_mma = more && ts * AB < ksteps;      // uniform
                     // this slot's MFMA operands arrive while its geometry is set up; the offsets of the
                     // next tap slot travel while this one is worked on
@@ -899,9 +904,6 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     else load_slot_offsets(tap0 + TP + MM::row(0, 0) / CCH, 0);
                     __builtin_amdgcn_sched_barrier(0);
 
-                    int kd[ND];
-#pragma unroll
-                    for (int a = 0; a < ND; ++a) kd[a] = sKd[min(tap, P.kV - 1) * ND + a];
                     TapGeo<T, ND> t;
                     tap_setup<T, ND>(P, ofs, ib, kd, t);
                     const bool slot_ok = valid && tap < P.kV;
@@ -927,53 +929,43 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     T sg[ND];
 #pragma unroll
                     for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= (T)P.in[0]) ? (T)1 : (T)0);
+                    const bool near = live && in_halo, far = live && !in_halo;
+                    // d(sample)/d(coordinate) of one channel from its corner values, times gcol
+                    auto coord_grad = [&](const T v[NC], T gv) {
+                        if constexpr (ND == 3) {
+                            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                            ga[0] += gv * (((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
+                                           ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh);
+                            ga[1] += gv * (((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
+                                           ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl);
+                            ga[2] += gv * (((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                           ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl);
+                        } else {
+                            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                            ga[0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
+                            ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
+                        }
+                    };
 #pragma unroll
                     for (int rr = 0; rr < RPS; ++rr) {
                         const int r = ts * RPS + rr;
                         const int cl = MM::row(r, q) % CCH;
                         const T gv = d[r];
                         if (cl >= nch) {
-                        } else if (live) {
+                        } else if (near) {
+                            // the reads go first: LDS operations complete in order, so the interpolation
+                            // gradient below waits for them only, not for the adds issued after them
                             T v[NC];
-                            if (in_halo) {
-                                // the reads go first: LDS operations complete in order, so the interpolation
-                                // gradient below waits for them only, not for the adds issued after them
-                                if constexpr (COORD) {
-                                    const T* ip = sIn + cl * P.hstride;
-#pragma unroll
-                                    for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
-                                }
-                                Cell* plane = sG + cl * P.hstride;
-                                const double gs = LdsCell<T>::pre(gv, scale);
-#pragma unroll
-                                for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
-                            } else {
-                                const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
-                                T* gc = gin + chan;
-#pragma unroll
-                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
-                                if constexpr (COORD) {
-                                    const T* ic = in + chan;
-#pragma unroll
-                                    for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
-                                }
-                            }
                             if constexpr (COORD) {
-                                if constexpr (ND == 3) {
-                                    const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh,
-                                            fw = t.f[2], gw = (T)1 - fw;
-                                    ga[0] += gv * (((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
-                                                   ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh);
-                                    ga[1] += gv * (((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
-                                                   ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl);
-                                    ga[2] += gv * (((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
-                                                   ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl);
-                                } else {
-                                    const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                                    ga[0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
-                                    ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
-                                }
+                                const T* ip = sIn + cl * P.hstride;
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
                             }
+                            Cell* plane = sG + cl * P.hstride;
+                            const double gs = LdsCell<T>::pre(gv, scale);
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+                            if constexpr (COORD) coord_grad(v, gv);
                         } else if (oor) {
                             const T av = gv > 0 ? gv : -gv;
 #pragma unroll
@@ -984,6 +976,27 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 #pragma unroll
                             for (int k = 0; k < MPR; ++k)
                                 d_next = MM::mma(a_cu[rr * MPR + k], BREG ? b_reg[ts * AB + rr * MPR + k] : b_cu[rr * MPR + k], d_next);
+                        }
+                    }
+                    if (__any(far)) {              // rare: samples that reach past the halo go to global memory
+#pragma unroll
+                        for (int rr = 0; rr < RPS; ++rr) {
+                            const int r = ts * RPS + rr;
+                            const int cl = MM::row(r, q) % CCH;
+                            if (far && cl < nch) {
+                                const T gv = d[r];
+                                const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
+                                T* gc = gin + chan;
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
+                                if constexpr (COORD) {
+                                    const T* ic = in + chan;
+                                    T v[NC];
+#pragma unroll
+                                    for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
+                                    coord_grad(v, gv);
+                                }
+                            }
                         }
                     }
                     if constexpr (COORD) {
