@@ -170,6 +170,44 @@ __device__ inline void tap_setup(const Params& P, const T offv[ND], const int ib
     }
 }
 
+// The same without corner indices (t.idx stays unset): for callers that sample from an LDS halo
+// and need global offsets only for the rare samples that reach past it (tap_corner_idx).
+template <typename T, int ND>
+__device__ inline void tap_setup_noidx(const Params& P, const T offv[ND], const int ib[ND], const int kd[ND],
+                                       TapGeo<T, ND>& t) {
+    bool inside = true;
+#pragma unroll
+    for (int a = 0; a < ND; ++a) {
+        const int size = P.in[slot<ND>(a)];
+        const T p = (T)(ib[a] + kd[a]) + offv[a];
+        t.p[a] = p;
+        inside = inside && (p > (T)-1) && (p < (T)size);
+        const int l = (int)p;
+        t.lo[a] = l;
+        t.hi[a] = (p >= (T)(size - 1) || p <= (T)0) ? l : l + 1;
+        t.f[a] = p - (T)l;
+    }
+    t.inside = inside;
+}
+template <typename T, int ND>
+__device__ inline void tap_corner_idx(const Params& P, TapGeo<T, ND>& t) {
+    if constexpr (ND == 3) {
+        const unsigned s1 = P.in[2], s2 = P.in[1] * P.in[2];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int l = (c & 4) ? t.hi[0] : t.lo[0], h = (c & 2) ? t.hi[1] : t.lo[1], w = (c & 1) ? t.hi[2] : t.lo[2];
+            t.idx[c] = t.inside ? (unsigned)l * s2 + (unsigned)h * s1 + (unsigned)w : 0u;
+        }
+    } else {
+        const unsigned s1 = P.in[2];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int h = (c & 2) ? t.hi[0] : t.lo[0], w = (c & 1) ? t.hi[1] : t.lo[1];
+            t.idx[c] = t.inside ? (unsigned)h * s1 + (unsigned)w : 0u;
+        }
+    }
+}
+
 // Interpolated value of one channel: lerp along w, then h, then l (reference order,
 // deform3d kernel.cu:48-56, deform2d_double kernel.cu:50-53).  `chan` points at the channel's
 // first voxel; `voff` are the corner offsets (possibly biased by the caller, see kernels).

@@ -651,8 +651,8 @@ template <typename T> struct LdsCell;
 template <> struct LdsCell<float> {
     typedef unsigned long long type;
     static constexpr double MAGIC = 6755399441055744.0;     // 1.5 * 2^52: low mantissa bits = integer value
-    __device__ static inline void add(type* p, float w, double gv_scaled) {
-        const double d = __builtin_fma((double)w, gv_scaled, MAGIC);
+    __device__ static inline void add(type* p, double w, double gv_scaled) {
+        const double d = __builtin_fma(w, gv_scaled, MAGIC);
         const long long bits = __double_as_longlong(d) - __double_as_longlong(MAGIC);
         (void)__hip_atomic_fetch_add(p, (type)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -905,7 +905,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     __builtin_amdgcn_sched_barrier(0);
 
                     TapGeo<T, ND> t;
-                    tap_setup<T, ND>(P, ofs, ib, kd, t);
+                    tap_setup_noidx<T, ND>(P, ofs, ib, kd, t);
                     const bool slot_ok = valid && tap < P.kV;
                     const bool live = slot_ok && t.inside;
                     T ga[ND];
@@ -923,6 +923,9 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                         const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
                         cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
                     }
+                    double cwd[NC];                // widened once per tap slot, used for every channel
+#pragma unroll
+                    for (int i = 0; i < NC; ++i) cwd[i] = (double)cw[i];
                     // out-of-range samples of the 3-D operator: +-|gcol| per axis; h and w are compared
                     // with the LENGTH extent
                     const bool oor = COORD && ND == 3 && slot_ok && !t.inside;
@@ -931,13 +934,14 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                     for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= (T)P.in[0]) ? (T)1 : (T)0);
                     const bool near = live && in_halo, far = live && !in_halo;
                     // d(sample)/d(coordinate) of one channel from its corner values, times gcol
+                    // (the w-lerps of the four (l, h) corner pairs are shared by the l and h derivatives)
                     auto coord_grad = [&](const T v[NC], T gv) {
                         if constexpr (ND == 3) {
                             const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
-                            ga[0] += gv * (((v[4] - v[0]) * gw + (v[5] - v[1]) * fw) * gh +
-                                           ((v[6] - v[2]) * gw + (v[7] - v[3]) * fw) * fh);
-                            ga[1] += gv * (((v[2] - v[0]) * gw + (v[3] - v[1]) * fw) * gl +
-                                           ((v[6] - v[4]) * gw + (v[7] - v[5]) * fw) * fl);
+                            const T c00 = v[0] * gw + v[1] * fw, c01 = v[2] * gw + v[3] * fw;
+                            const T c10 = v[4] * gw + v[5] * fw, c11 = v[6] * gw + v[7] * fw;
+                            ga[0] += gv * ((c10 - c00) * gh + (c11 - c01) * fh);
+                            ga[1] += gv * ((c01 - c00) * gl + (c11 - c10) * fl);
                             ga[2] += gv * (((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
                                            ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl);
                         } else {
@@ -964,7 +968,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                             Cell* plane = sG + cl * P.hstride;
                             const double gs = LdsCell<T>::pre(gv, scale);
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cw[i], gs);
+                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cwd[i], gs);
                             if constexpr (COORD) coord_grad(v, gv);
                         } else if (oor) {
                             const T av = gv > 0 ? gv : -gv;
@@ -979,6 +983,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                         }
                     }
                     if (__any(far)) {              // rare: samples that reach past the halo go to global memory
+                        tap_corner_idx<T, ND>(P, t);
 #pragma unroll
                         for (int rr = 0; rr < RPS; ++rr) {
                             const int r = ts * RPS + rr;
@@ -988,7 +993,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                                 const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
                                 T* gc = gin + chan;
 #pragma unroll
-                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], cw[i] * gv);
+                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], (T)cwd[i] * gv);
                                 if constexpr (COORD) {
                                     const T* ic = in + chan;
                                     T v[NC];
