@@ -314,10 +314,16 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     const dim3 tgrid((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N), tblock(32, 8);
 
     // 1) one kernel: scatter privatised in LDS + coordinate gradient from an LDS input halo
+    // A halo of up to FUSED_HS cells gets the variant with that compile-time plane stride (the four
+    // planes of either kind then lie within the 64 KB reach of an LDS instruction's offset field).
+    constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
     Params Ph = P;
-    if (scatter_in_lds() && fused_coord() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T)) &&
-        (scatter_budget() - (size_t)Ph.hvol * 4 - (size_t)P.kV * ND * 4) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4) {
+    const bool planned = scatter_in_lds() && fused_coord() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T));
+    const size_t tables = planned ? (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4 : 0;
+    const bool fixed = planned && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
+    if (planned && (fixed || (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4)) {
         Ph.cchunk = 4;
+        if (fixed) Ph.hstride = FUSED_HS;
         const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
@@ -341,10 +347,14 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         }
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG, (unsigned)csplit);
         // grad_output operand held in registers when its reduction steps fit (M <= 64 float, 128 double)
-        if ((P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true>, "backward_input_halo_kernel", hgrid, WGH, lds,
-                               s, Ph, in, off, wt, gout, wmax, gin, goff);
-        return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
+        const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32;
+        if (fixed && breg)
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true, FUSED_HS>, "backward_input_halo_kernel", hgrid, WGH,
+                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff);
+        if (fixed)
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false, FUSED_HS>, "backward_input_halo_kernel", hgrid, WGH,
+                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff);
+        return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
                            in, off, wt, gout, wmax, gin, goff);
     }
 
@@ -375,10 +385,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)
-            return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff);
         if (Ph.cchunk == 4)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }

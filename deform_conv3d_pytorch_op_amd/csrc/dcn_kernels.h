@@ -709,7 +709,9 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // chunk after chunk (the first chunk stores).  dynamic LDS then adds CCH * hstride * sizeof(T).
 // BREG = true (host: at most NS * 8 reduction steps, i.e. M <= 64 for float) keeps this lane's
 // grad_output values -- the B operand, the same for every tap and channel chunk -- in registers.
-template <typename T, int ND, int CCH, bool COORD, bool BREG>
+// HS > 0 fixes the plane stride at compile time (the host then plans with hstride = HS): the plane
+// of a channel becomes an immediate offset of the LDS instructions instead of address arithmetic.
+template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS>
 __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
@@ -724,9 +726,10 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     constexpr int NS = NACC / RPS;                      // tap slots per lane and pass
     static_assert(TN % CCH == 0 && CCH % 4 == 0 && NACC % RPS == 0, "unsupported channel chunk");
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int hs = HS ? HS : P.hstride;
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
-    T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * P.hstride);                        // [CCH][hstride] if COORD
-    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * P.hstride : 0));   // [hvol]
+    T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * hs);                               // [CCH][hstride] if COORD
+    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
     int* sKd = reinterpret_cast<int*>(sTab + P.hvol);                                   // [kV][ND]: tap * dilation per axis
     __shared__ float sRed[WAVESH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -812,7 +815,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
             const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
-                for (int v = threadIdx.x; v < P.hvol; v += WGH) sG[c * P.hstride + v] = 0;      // all-zero bits in either cell type
+                for (int v = threadIdx.x; v < P.hvol; v += WGH) sG[c * hs + v] = 0;      // all-zero bits in either cell type
             if constexpr (COORD) halo_stage<T>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
 
@@ -933,6 +936,12 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 #pragma unroll
                     for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= (T)P.in[0]) ? (T)1 : (T)0);
                     const bool near = live && in_halo, far = live && !in_halo;
+                    // corner cells of channel 0; the other channels are an immediate offset away when the
+                    // plane stride is a compile-time constant
+                    Cell* g_cell[NC];
+                    const T* in_cell[NC];
+#pragma unroll
+                    for (int i = 0; i < NC; ++i) { g_cell[i] = sG + lidx[i]; in_cell[i] = sIn + lidx[i]; }
                     // d(sample)/d(coordinate) of one channel from its corner values, times gcol
                     // (the w-lerps of the four (l, h) corner pairs are shared by the l and h derivatives)
                     auto coord_grad = [&](const T v[NC], T gv) {
@@ -961,14 +970,12 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                             // gradient below waits for them only, not for the adds issued after them
                             T v[NC];
                             if constexpr (COORD) {
-                                const T* ip = sIn + cl * P.hstride;
 #pragma unroll
-                                for (int i = 0; i < NC; ++i) v[i] = ip[lidx[i]];
+                                for (int i = 0; i < NC; ++i) v[i] = in_cell[i][cl * hs];
                             }
-                            Cell* plane = sG + cl * P.hstride;
                             const double gs = LdsCell<T>::pre(gv, scale);
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(plane + lidx[i], cwd[i], gs);
+                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(g_cell[i] + cl * hs, cwd[i], gs);
                             if constexpr (COORD) coord_grad(v, gv);
                         } else if (oor) {
                             const T av = gv > 0 ? gv : -gv;
@@ -1032,7 +1039,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                 const unsigned gv = sTab[v];
                 if (gv == ~0u) continue;            // halo cell outside the volume: never touched
                 for (int c = 0; c < nch; ++c) {
-                    const Cell cell = sG[c * P.hstride + v];
+                    const Cell cell = sG[c * hs + v];
                     if (cell != (Cell)0)
                         atomic_add(gin + ((size_t)n * P.C_in + cc0 + c) * P.inV + gv, (T)LdsCell<T>::value(cell, inv_scale));
                 }
