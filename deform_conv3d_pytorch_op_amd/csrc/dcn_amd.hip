@@ -249,18 +249,19 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     if (MT <= 2 && wide_forward()) {
         Params Pw = P;
         if (plan_halo<T, ND>(Pw, 144 * 1024, 1 << 30, sizeof(T), 16) &&
+            (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks <= 0x7fffffffLL &&
             (wide_forward() == 2 || (Pw.cchunk >= 8 && (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks >= cu_count()))) {
             const size_t lds = (size_t)Pw.cchunk * Pw.hstride * sizeof(T) + (size_t)Pw.hvol * 4;
-            const dim3 grid((unsigned)Pw.N * Pw.tiles, (unsigned)Pw.G * Pw.mchunks);
+            const dim3 grid((unsigned)Pw.N * Pw.tiles * Pw.G * Pw.mchunks);
             if (MT == 1) return launch_halo(forward_halo_kernel<T, ND, 1, 16>, "forward_halo_kernel", grid, 1024, lds, s, Pw, in, off, wt, bias, out);
             return launch_halo(forward_halo_kernel<T, ND, 2, 16>, "forward_halo_kernel", grid, 1024, lds, s, Pw, in, off, wt, bias, out);
         }
     }
     bool tiled = plan_halo<T, ND>(P, LDS_BUDGET);
     if ((!tiled || P.cchunk < 8) && LDS_BUDGET < 144 * 1024) tiled = plan_halo<T, ND>(P, 144 * 1024) || tiled;
-    if (tiled) {
+    if (tiled && (long long)P.N * P.tiles * P.G * P.mchunks <= 0x7fffffffLL) {
         const size_t lds = (size_t)P.cchunk * P.hstride * sizeof(T) + (size_t)P.hvol * 4;
-        const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
+        const dim3 grid((unsigned)P.N * P.tiles * P.G * P.mchunks);
         switch (MT) {
             case 1: return launch_halo(forward_halo_kernel<T, ND, 1, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
             case 2: return launch_halo(forward_halo_kernel<T, ND, 2, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
@@ -321,7 +322,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     const bool planned = scatter_in_lds() && fused_coord() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T));
     const size_t tables = planned ? (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4 : 0;
     const bool fixed = planned && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
-    if (planned && (fixed || (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4)) {
+    if (planned && (long long)Ph.N * Ph.tiles * Ph.DG * 4 <= 0x7fffffffLL && (fixed || (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4)) {
         Ph.cchunk = 4;
         if (fixed) Ph.hstride = FUSED_HS;
         const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
@@ -345,17 +346,17 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fb), dim3(256), 0, s, goff, nel);
             if (int rc = check_launch("fill_zero_kernel")) return rc;
         }
-        const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG, (unsigned)csplit);
+        const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG * csplit);
         // grad_output operand held in registers when its reduction steps fit (M <= 64 float, 128 double)
         const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32;
         if (fixed && breg)
             return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true, FUSED_HS>, "backward_input_halo_kernel", hgrid, WGH,
-                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff);
+                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit);
         if (fixed)
             return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false, FUSED_HS>, "backward_input_halo_kernel", hgrid, WGH,
-                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff);
+                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit);
         return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
-                           in, off, wt, gout, wmax, gin, goff);
+                           in, off, wt, gout, wmax, gin, goff, csplit);
     }
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
@@ -363,6 +364,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
     Ph = P;
     bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
+    if (halo && (long long)Ph.N * Ph.tiles * Ph.DG > 0x7fffffffLL) halo = false;
     if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
         const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4 - (size_t)P.kV * ND * 4) / ((size_t)Ph.hstride * 8);
         if (fit >= 8) Ph.cchunk = 8;
@@ -382,14 +384,14 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         if (int rc = check_launch("backward_data_kernel")) return rc;
         const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
-        const dim3 hgrid((unsigned)Ph.N * Ph.tiles, (unsigned)Ph.DG);
+        const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG);
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)
             return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
-                               Ph, in, off, wt, gout, wmax, gin, nogoff);
+                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1);
         if (Ph.cchunk == 4)
             return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
-                               Ph, in, off, wt, gout, wmax, gin, nogoff);
+                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }
     // halo does not fit in LDS: scatter with global atomics on the channels-last copy

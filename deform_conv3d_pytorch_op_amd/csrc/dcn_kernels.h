@@ -122,6 +122,17 @@ constexpr int WGH = 512;
 constexpr int WAVESH = WGH / 64;
 constexpr int MAX_HVOL = 6144;     // halo voxels per workgroup tile (the LDS table holds one entry each)
 
+// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin by launch order.  This
+// maps the launch index of a 1-D grid to a logical index such that each XCD works through one
+// contiguous range of logical indices: neighbouring tiles, and the workgroups that share a tile,
+// then meet in the same L2 at about the same time.
+__device__ inline unsigned xcd_contiguous(unsigned launch_idx, unsigned total) {
+    constexpr unsigned XCDS = 8;
+    const unsigned xcd = launch_idx % XCDS, slot = launch_idx / XCDS;
+    const unsigned qq = total / XCDS, rr = total % XCDS;
+    return xcd * qq + (xcd < rr ? xcd : rr) + slot;
+}
+
 template <int ND>
 struct TileGeo {
     int n;              // sample
@@ -239,7 +250,7 @@ __device__ inline bool halo_corners(const Params& P, const int hb[ND], const Tap
 
 // Forward with the input halo in LDS.  Same contraction and lane roles as forward_kernel; the
 // sampled value of lane (j, q) is the MFMA B operand B[k = q][col = j].
-// grid.x = N * tiles (3-D blocks of positions), grid.y = G * mchunks, NW wavefronts per workgroup
+// 1-D grid of N * tiles (3-D blocks of positions) * G * mchunks, NW wavefronts per workgroup
 // (16 when the accumulators are few enough for 128 registers: the larger block shares each staged
 // halo between twice the positions); dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4.
 template <typename T, int ND, int MT, int NW>
@@ -253,10 +264,13 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)P.cchunk * P.hstride);   // [hvol]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
-    const int g = blockIdx.y / P.mchunks, mchunk = blockIdx.y % P.mchunks;
+    // 1-D grid of N * tiles * G * mchunks workgroups; those of one tile are neighbours
+    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+    const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
+    const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
 
     TileGeo<ND> tg;
-    tile_decode<ND>(P, blockIdx.x, tg);
+    tile_decode<ND>(P, wg / (unsigned)(P.G * P.mchunks), tg);
     const int n = tg.n;
     int o[ND], ib[ND];
     unsigned pos;
@@ -700,7 +714,7 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // atomics.  After all taps the planes are added to grad_input with one hardware float atomic per
 // touched halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that
 // reach past the halo use global atomics directly.
-// grid.x = N * tiles, grid.y = DG; dynamic LDS = CCH * hstride * 8 + hvol * 4 + kV * ND * 4 bytes.
+// dynamic LDS = CCH * hstride * 8 + hvol * 4 + kV * ND * 4 bytes.
 // COORD = true additionally stages the same CCH input channels over the halo (float planes) and
 // computes grad_offset in the same pass over the grad-column values (col2im_offset of the
 // reference, deform3d kernel.cu:386-483 incl. the out-of-range branches :470-481, 2-D
@@ -717,7 +731,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                                                                   const T* __restrict__ Wt,
                                                                   const T* __restrict__ gout,
                                                                   const float* __restrict__ wmax,
-                                                                  T* __restrict__ gin, T* __restrict__ goff) {
+                                                                  T* __restrict__ gin, T* __restrict__ goff, int csplit) {
     using MM = Mma<T>;
     using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
@@ -734,14 +748,17 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     __shared__ float sRed[WAVESH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
-    const int dg = blockIdx.y;
-    // gridDim.z workgroups share one (tile, deformable group): workgroup z takes every gridDim.z-th
-    // channel chunk (finer work items shorten the last, partly filled round of workgroups).  Their
-    // grad_offset contributions then meet through float atomics on a zero-filled buffer.
-    const int csplit = gridDim.z, cz = blockIdx.z;
+    // 1-D grid of DG * N * tiles * csplit workgroups.  csplit workgroups share one (tile, deformable
+    // group): workgroup cz takes every csplit-th channel chunk (finer work items shorten the last,
+    // partly filled round of workgroups).  Their grad_offset contributions then meet through float
+    // atomics on a zero-filled buffer.
+    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int cz = wg % (unsigned)csplit;
+    const unsigned nt = (unsigned)P.N * P.tiles;
+    const int dg = (wg / csplit) / nt;
 
     TileGeo<ND> tg;
-    tile_decode<ND>(P, blockIdx.x, tg);
+    tile_decode<ND>(P, (wg / csplit) % nt, tg);
     const int n = tg.n;
     int o[ND], ib[ND];
     unsigned pos;
