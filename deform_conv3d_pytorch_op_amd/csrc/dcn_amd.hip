@@ -241,8 +241,21 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     fwd_weight_pad<T>(P.M, P.Cg, MT, P.mchunks, P.Mp, P.Cgp);
     if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
     T* wt = static_cast<T*>(ws);
-    if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     const int TN = Mma<T>::TN;
+    // Small position counts with many output channels: fewer row tiles per wavefront (more output
+    // channel chunks, each sampling for itself) until there is a workgroup for every CU.
+    {
+        Params Pt = P;
+        const long long tiles = plan_halo<T, ND>(Pt, 144 * 1024) ? (long long)Pt.N * Pt.tiles
+                                                                  : (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN));
+        const int mtiles = (P.M + TN - 1) / TN;
+        while (MT > 1 && tiles * P.G * P.mchunks < cu_count()) {
+            MT /= 2;
+            P.mchunks = (mtiles + MT - 1) / MT;
+        }
+        P.Mp = P.mchunks * MT * TN;
+    }
+    if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     // Few accumulators (MT <= 2): one 1024-thread workgroup per CU with the whole LDS, if its larger
     // halo fits and leaves 8 channels per pass.  Otherwise 512 threads: two workgroups per CU when
     // that still leaves 8 channels per LDS pass, else one large one.
