@@ -458,7 +458,7 @@ int launch_bwd_weight(const Params& P, const T* in_cl, const T* off, const T* go
             return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
         }
     }
-    const dim3 grid((unsigned)P.nsplit, (unsigned)P.kV, (unsigned)(P.nctiles * P.mchunks));
+    const dim3 grid((unsigned)P.nsplit * P.kV * P.nctiles * P.mchunks);
     hipLaunchKernelGGL(kern, grid, dim3(WG), lds, s, P, in_cl, off, gout_cl, partial);
     return check_launch("backward_weight_kernel");
 }

@@ -1079,7 +1079,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 // over position slabs independently (no workgroup barriers), so the [MT*TN x TN] accumulator
 // stays in registers; each workgroup writes one partial tile per split and a small second kernel
 // sums the splits into grad_weight (deterministic, no atomics).
-// grid.x = nsplit, grid.y = kV, grid.z = nctiles * mchunks; dynamic LDS = WAVES * MT*TN * (TN+1) * sizeof(T).
+// dynamic LDS = WAVES * MT*TN * (TN+1) * sizeof(T).
 template <typename T, int ND, int MT>
 __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* __restrict__ in_cl,
                                                              const T* __restrict__ off,
@@ -1093,9 +1093,14 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
 
-    const int tap = blockIdx.y;
-    const int mchunk = blockIdx.z % P.mchunks;
-    int z = blockIdx.z / P.mchunks;
+    // 1-D grid of nctiles * mchunks * nsplit * kV workgroups in an XCD-contiguous order with the tap
+    // fastest: the workgroups that gather around the same positions and channels share an L2
+    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int tap = wg % (unsigned)P.kV;
+    const int split = (wg / (unsigned)P.kV) % (unsigned)P.nsplit;
+    const unsigned zz = (wg / (unsigned)P.kV) / (unsigned)P.nsplit;
+    const int mchunk = zz % P.mchunks;
+    int z = zz / P.mchunks;
     // locate channel tile z: segments are the intersections of convolution groups with deformable groups
     int g = 0, dg = 0, c0 = 0, ce = 0;
     bool found = false;
@@ -1135,7 +1140,7 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 
     const int slabs_per_sample = (P.outV + TN - 1) / TN;
     const int nslabs = P.N * slabs_per_sample;
-    for (int slab = blockIdx.x * WAVES + wave; slab < nslabs; slab += gridDim.x * WAVES) {
+    for (int slab = split * WAVES + wave; slab < nslabs; slab += P.nsplit * WAVES) {
         const int n = slab / slabs_per_sample;
         const unsigned p0 = (unsigned)(slab % slabs_per_sample) * TN;
         const unsigned pos = p0 + j;
@@ -1217,7 +1222,7 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
         for (int r = 0; r < MM::NACC; ++r)
             sAcc[((size_t)wave * MT * TN + mt * TN + MM::row(r, q)) * LDA + j] = acc[mt][r];
     __syncthreads();
-    T* pt = partial + ((size_t)blockIdx.x * P.kV + tap) * P.C_out * P.Cg;
+    T* pt = partial + ((size_t)split * P.kV + tap) * P.C_out * P.Cg;
     for (int e = threadIdx.x; e < MT * TN * TN; e += WG) {
         const int mr = e / TN, cc = e % TN;
         const int m = m_base + mr, c = c0 + cc;
