@@ -911,6 +911,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
                 if constexpr (!BREG) { if (more && ksteps > NS * AB) gemm_tail(d_next, wnext, NS * AB); }
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
+                    // slots past the last tap (only in the last pass, which feeds no further MFMAs)
+                    if (tap0 + MM::row(ts * RPS, 0) / CCH >= P.kV) continue;
                     const int tap = tap0 + MM::row(ts * RPS, q) / CCH;
                     T a_cu[AB], b_cu[AB], ofs[ND];
                     int kd[ND];
