@@ -33,9 +33,9 @@ PEAK_HBM_GBS = 8000.0
 # the summary with the commands is profiles/c4_deform3d_f32_fwd_bwd_kernels.md.  Only for configurations
 # that were profiled; otherwise `traffic` is null.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 2.603e9,
-    ("c4", "backward_input_offset"): 10.26e9,
-    ("c4", "backward_weight"): 7.363e9,
+    ("c4", "forward"): 0.524e9,
+    ("c4", "backward_input_offset"): 1.981e9,
+    ("c4", "backward_weight"): 1.349e9,
 }
 
 # name: (nd, N, C_in, C_out, in, k, stride, pad, dil, cpg, groups, offset scale / dist, dtype)

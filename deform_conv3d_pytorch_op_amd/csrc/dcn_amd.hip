@@ -449,7 +449,7 @@ void bww_plan(const Params& Pin, int& MT, int& mchunks, int& nct, int& nsplit) {
 template <typename T, int ND, int MT>
 int launch_bwd_weight(const Params& P, const T* in_cl, const T* off, const T* gout_cl, T* partial, hipStream_t s) {
     const int TN = Mma<T>::TN;
-    const size_t lds = (size_t)WAVES * MT * TN * (TN + 1) * sizeof(T);
+    const size_t lds = (size_t)WAVES * TN * (TN + 1) * sizeof(T);
     auto kern = backward_weight_kernel<T, ND, MT>;
     if (lds > 48 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -1081,7 +1081,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
 // over position slabs independently (no workgroup barriers), so the [MT*TN x TN] accumulator
 // stays in registers; each workgroup writes one partial tile per split and a small second kernel
 // sums the splits into grad_weight (deterministic, no atomics).
-// dynamic LDS = WAVES * MT*TN * (TN+1) * sizeof(T).
+// dynamic LDS = WAVES * TN * (TN+1) * sizeof(T).
 template <typename T, int ND, int MT>
 __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* __restrict__ in_cl,
                                                              const T* __restrict__ off,
@@ -1091,7 +1091,7 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
     __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // corner voxel index * C_in, 0 when the sample is dead
     __shared__ __align__(16) T sF[WAVES][TN][4];             // f[ND]; [3] = 1 when the sample is live
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sAcc = reinterpret_cast<T*>(smem_raw);                // [WAVES][MT*TN][TN + 1]: the wavefronts' partial tiles
+    T* sAcc = reinterpret_cast<T*>(smem_raw);                // [WAVES][TN][TN + 1]: the wavefronts' partial tiles, one row tile at a time
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
 
@@ -1217,22 +1217,25 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
     // The four wavefronts' tiles are summed through LDS and the workgroup writes ONE partial tile
     // to its own slot of the workspace: partial[split][tap][g*M + m][c_local].  (Float atomics
     // straight into grad_weight cost 1.6 ms at 64x64x27 weights: a few hundred writers per address.)
+    // One row tile at a time, so that the LDS footprint (and with it the number of resident
+    // workgroups that hide the gather latency) does not grow with MT.
     constexpr int LDA = TN + 1;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int r = 0; r < MM::NACC; ++r)
-            sAcc[((size_t)wave * MT * TN + mt * TN + MM::row(r, q)) * LDA + j] = acc[mt][r];
-    __syncthreads();
     T* pt = partial + ((size_t)split * P.kV + tap) * P.C_out * P.Cg;
-    for (int e = threadIdx.x; e < MT * TN * TN; e += WG) {
-        const int mr = e / TN, cc = e % TN;
-        const int m = m_base + mr, c = c0 + cc;
-        if (m < P.M && c < ce) {
-            T sum = 0;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) sum += sAcc[((size_t)w * MT * TN + mr) * LDA + cc];
-            pt[((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)] = sum;
+    for (int mt = 0; mt < MT; ++mt) {
+        if (mt) __syncthreads();                    // readers of the previous tile are done
+#pragma unroll
+        for (int r = 0; r < MM::NACC; ++r) sAcc[((size_t)wave * TN + MM::row(r, q)) * LDA + j] = acc[mt][r];
+        __syncthreads();
+        for (int e = threadIdx.x; e < TN * TN; e += WG) {
+            const int mr = e / TN, cc = e % TN;
+            const int m = m_base + mt * TN + mr, c = c0 + cc;
+            if (m < P.M && c < ce) {
+                T sum = 0;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) sum += sAcc[((size_t)w * TN + mr) * LDA + cc];
+                pt[((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)] = sum;
+            }
         }
     }
 }
