@@ -1176,36 +1176,39 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
         // multiplied, the geometry record, the corner values and the grad_output rows of step ks + 1
         // are already in flight
         constexpr int NK = TN / KL;
-        T cn[NC], an[MT], fn[ND];                   // "next" step
-        bool lvn, okn;
-        auto fetch = [&](int ks) {
+        constexpr int DEPTH = 1;                    // steps in flight ahead of the one being multiplied (2 costs a wavefront of occupancy and is slower)
+        T cn[DEPTH][NC], an[DEPTH][MT], fn[DEPTH][ND];
+        bool lvn[DEPTH], okn[DEPTH];
+        auto fetch = [&](int ks, int slot_) {
             const int pp = ks * KL + q;             // position of the slab this lane group works on
             unsigned ix[NC];
 #pragma unroll
             for (int i = 0; i < NC; ++i) ix[i] = sIdx[wave][pp][i];
 #pragma unroll
-            for (int a_ = 0; a_ < ND; ++a_) fn[a_] = sF[wave][pp][a_];
-            lvn = sF[wave][pp][3] != (T)0;
+            for (int a_ = 0; a_ < ND; ++a_) fn[slot_][a_] = sF[wave][pp][a_];
+            lvn[slot_] = sF[wave][pp][3] != (T)0;
             const unsigned pg = min(p0 + (unsigned)pp, P.outV - 1);
-            okn = p0 + (unsigned)pp < P.outV;
+            okn[slot_] = p0 + (unsigned)pp < P.outV;
             const T* grow = go_n + (size_t)pg * P.C_out;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) an[mt] = grow[mrow[mt]];      // A[row = m][k = position]; legal for every lane
-            load_corners<T, ND>(in_n, ix, cn);                           // dead samples read voxel 0
+            for (int mt = 0; mt < MT; ++mt) an[slot_][mt] = grow[mrow[mt]];   // A[row = m][k = position]; legal for every lane
+            load_corners<T, ND>(in_n, ix, cn[slot_]);                         // dead samples read voxel 0
         };
-        fetch(0);
+#pragma unroll
+        for (int d0 = 0; d0 < DEPTH; ++d0) fetch(d0, d0);
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks) {
+            const int sl = ks % DEPTH;
             T cc[NC], ac[MT], fc[ND];
 #pragma unroll
-            for (int i = 0; i < NC; ++i) cc[i] = cn[i];
+            for (int i = 0; i < NC; ++i) cc[i] = cn[sl][i];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) ac[mt] = an[mt];
+            for (int mt = 0; mt < MT; ++mt) ac[mt] = an[sl][mt];
 #pragma unroll
-            for (int a_ = 0; a_ < ND; ++a_) fc[a_] = fn[a_];
-            const bool lvc = lvn, okc = okn;
-            if (ks + 1 < NK) fetch(ks + 1);
-            __builtin_amdgcn_sched_barrier(0);      // next step's loads are issued before this step's arithmetic
+            for (int a_ = 0; a_ < ND; ++a_) fc[a_] = fn[sl][a_];
+            const bool lvc = lvn[sl], okc = okn[sl];
+            if (ks + DEPTH < NK) fetch(ks + DEPTH, sl);
+            __builtin_amdgcn_sched_barrier(0);      // later steps' loads are issued before this step's arithmetic
             const T v = interp<T, ND>(cc, fc);
             const T b = (lvc && chan_ok) ? v : (T)0;                                   // B[k = position][col = channel j]
 #pragma unroll
@@ -1214,9 +1217,6 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
         }
     }
 
-    // The four wavefronts' tiles are summed through LDS and the workgroup writes ONE partial tile
-    // to its own slot of the workspace: partial[split][tap][g*M + m][c_local].  (Float atomics
-    // straight into grad_weight cost 1.6 ms at 64x64x27 weights: a few hundred writers per address.)
     // One row tile at a time, so that the LDS footprint (and with it the number of resident
     // workgroups that hide the gather latency) does not grow with MT.
     constexpr int LDA = TN + 1;
