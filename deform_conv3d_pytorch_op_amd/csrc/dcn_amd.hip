@@ -137,6 +137,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
+//   DCN_FUSED_WAVES=4      fused backward kernel with four wavefronts per workgroup even where eight fit
 static size_t env_kb(const char* name, int dflt) {
     const char* e = getenv(name);
     const int v = e ? atoi(e) : dflt;
@@ -166,6 +167,10 @@ static int wide_forward() {      // 0 never, 1 when it pays, 2 whenever the halo
     }();
     return v;
 }
+static int fused_first_waves() {
+    static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : 8; }();
+    return v;
+}
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
     return v != 0;
@@ -183,12 +188,27 @@ int halo_margin() {
 }
 
 template <typename T, int ND>
-bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH) {
+bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH,
+               bool smallest_halo = false) {
     const int npos = waves * Mma<T>::TN;        // positions per workgroup, one column tile per wavefront
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
     else         { td[2] = 16; td[1] = npos / 16; }
     const int m = halo_margin();
+    if (smallest_halo) {
+        // the block shape (powers of two, at least 4 positions along the fastest axis) with the
+        // smallest halo: strided geometries want blocks that are short along the strided axes
+        long long best = -1;
+        for (int a = 1; a <= npos; a *= 2)
+            for (int b = 1; a * b <= npos; b *= 2) {
+                const int c = npos / (a * b);
+                if (c < 4 || (ND == 2 && a != 1)) continue;
+                const int cand[3] = {a, b, c};
+                long long hv = 1;
+                for (int x = 3 - ND; x < 3; ++x) hv *= (cand[x] - 1) * P.stride[x] + (P.k[x] - 1) * P.dil[x] + 1 + 2 * m;
+                if (best < 0 || hv < best) { best = hv; td[0] = a; td[1] = b; td[2] = c; }
+            }
+    }
     long long hvol = 1, tiles = 1;
     for (int a = 0; a < 3; ++a) {
         P.tdim[a] = td[a];
@@ -330,15 +350,19 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     // 1) one kernel: scatter privatised in LDS + coordinate gradient from an LDS input halo
     // A halo of up to FUSED_HS cells gets the variant with that compile-time plane stride (the four
     // planes of either kind then lie within the 64 KB reach of an LDS instruction's offset field).
+    // Eight wavefronts per workgroup; four (half the positions, in the block shape with the smallest
+    // halo) where only that fits, e.g. under stride 2.
     constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
-    Params Ph = P;
-    const bool planned = scatter_in_lds() && fused_coord() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T));
-    const size_t tables = planned ? (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4 : 0;
-    const bool fixed = planned && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
-    if (planned && (long long)Ph.N * Ph.tiles * Ph.DG * 4 <= 0x7fffffffLL && (fixed || (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 4)) {
+    for (int nw = fused_first_waves(); nw >= 4 && scatter_in_lds() && fused_coord(); nw /= 2) {
+        Params Ph = P;
+        if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T), nw, nw != 8)) continue;
+        const size_t tables = (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
+        const bool fixed = Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
+        if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
+        if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) < 4) continue;
         Ph.cchunk = 4;
         if (fixed) Ph.hstride = FUSED_HS;
-        const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
+        const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + tables;
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
         // wastes least of the last round (one workgroup per CU at this LDS size)
@@ -362,20 +386,24 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG * csplit);
         // grad_output operand held in registers when its reduction steps fit (M <= 64 float, 128 double)
         const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32;
-        if (fixed && breg)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true, FUSED_HS>, "backward_input_halo_kernel", hgrid, WGH,
-                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit);
-        if (fixed)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false, FUSED_HS>, "backward_input_halo_kernel", hgrid, WGH,
-                               lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit);
-        return launch_halo(backward_input_halo_kernel<T, ND, 4, true, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s, Ph,
-                           in, off, wt, gout, wmax, gin, goff, csplit);
+#define DCN_LAUNCH_FUSED(BREG_, HS_, NW_)                                                                              \
+    launch_halo(backward_input_halo_kernel<T, ND, 4, true, BREG_, HS_, NW_>, "backward_input_halo_kernel", hgrid, NW_ * 64, \
+                lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit)
+        if (nw == 8) {
+            if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 8);
+            if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 8);
+            return DCN_LAUNCH_FUSED(false, 0, 8);
+        }
+        if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 4);
+        if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 4);
+        return DCN_LAUNCH_FUSED(false, 0, 4);
+#undef DCN_LAUNCH_FUSED
     }
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
     hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
-    Ph = P;
+    Params Ph = P;
     bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
     if (halo && (long long)Ph.N * Ph.tiles * Ph.DG > 0x7fffffffLL) halo = false;
     if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
@@ -400,10 +428,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG);
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)
-            return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false, 0, WAVESH>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff, 1);
         if (Ph.cchunk == 4)
-            return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false, 0>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
+            return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false, 0, WAVESH>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
                                Ph, in, off, wt, gout, wmax, gin, nogoff, 1);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }

@@ -723,10 +723,11 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // chunk after chunk (the first chunk stores).  dynamic LDS then adds CCH * hstride * sizeof(T).
 // BREG = true (host: at most NS * 8 reduction steps, i.e. M <= 64 for float) keeps this lane's
 // grad_output values -- the B operand, the same for every tap and channel chunk -- in registers.
+// NW wavefronts per workgroup (8; 4 where only a smaller block of positions has a halo that fits).
 // HS > 0 fixes the plane stride at compile time (the host then plans with hstride = HS): the plane
 // of a channel becomes an immediate offset of the LDS instructions instead of address arithmetic.
-template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS>
-__global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
+template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW>
+__global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
                                                                   const T* __restrict__ gout,
@@ -745,7 +746,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * hs);                               // [CCH][hstride] if COORD
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
     int* sKd = reinterpret_cast<int*>(sTab + P.hvol);                                   // [kV][ND]: tap * dilation per axis
-    __shared__ float sRed[WAVESH];
+    constexpr int WGS = NW * 64;                        // threads per workgroup
+    __shared__ float sRed[NW];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     // 1-D grid of DG * N * tiles * csplit workgroups.  csplit workgroups share one (tile, deformable
@@ -765,8 +767,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
     const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
-    halo_table<ND>(P, tg, sTab);                   // visible after the first barrier below
-    for (int tp = threadIdx.x; tp < P.kV; tp += WGH) {      // taps differ between lanes here: a table replaces the divisions
+    halo_table<ND, WGS>(P, tg, sTab);                   // visible after the first barrier below
+    for (int tp = threadIdx.x; tp < P.kV; tp += WGS) {      // taps differ between lanes here: a table replaces the divisions
         int kk[ND];
         decode_tap<ND>(P, tp, kk);
 #pragma unroll
@@ -821,7 +823,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
         __syncthreads();
         float smax = 0.f;
 #pragma unroll
-        for (int w8 = 0; w8 < WAVESH; ++w8) smax = fmaxf(smax, sRed[w8]);
+        for (int w8 = 0; w8 < NW; ++w8) smax = fmaxf(smax, sRed[w8]);
         int ex = 0;
         const float bound = 8.f * wmax[0] * smax;
         if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
@@ -832,8 +834,8 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
             const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
-                for (int v = threadIdx.x; v < P.hvol; v += WGH) sG[c * hs + v] = 0;      // all-zero bits in either cell type
-            if constexpr (COORD) halo_stage<T>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
+                for (int v = threadIdx.x; v < P.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
+            if constexpr (COORD) halo_stage<T, WGS>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
 
             // Grad-column tile of a pass: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past
@@ -1054,7 +1056,7 @@ __global__ __launch_bounds__(WGH) void backward_input_halo_kernel(Params P, cons
             }
             first_chunk = false;
             __syncthreads();                        // all LDS adds of this chunk have landed
-            for (int v = threadIdx.x; v < P.hvol; v += WGH) {
+            for (int v = threadIdx.x; v < P.hvol; v += WGS) {
                 const unsigned gv = sTab[v];
                 if (gv == ~0u) continue;            // halo cell outside the volume: never touched
                 for (int c = 0; c < nch; ++c) {
