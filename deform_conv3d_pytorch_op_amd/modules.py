@@ -13,6 +13,11 @@ Initialisation: the reference draws Kaiming-normal (fan_out) and then overwrites
 the constant 1 (deform_conv3d_model.py:38-39); this keeps the Kaiming draw, which is what the
 float 2-D package does (deform2d ... :29).  Bias ~ U(-0.1, 0.1) as in the reference (:42).
 `device` and `dtype` are extra keyword arguments (the reference hard-codes cuda float / double).
+
+`ConvOffset{2,3}dPack` additionally own the plain convolution that the reference's callers put in
+front of the layer to produce the offsets (deform3d/test_model.py:18-30, deform2d/test_model.py:19-29):
+`nn.Conv{2,3}d(in_channels, in_channels // channel_per_group * nd * prod(kernel), kernel, stride,
+padding, bias=False)` on the same input; forward takes the input alone.
 """
 import torch
 import torch.nn as nn
@@ -59,6 +64,36 @@ class _ConvOffsetNd(nn.Module):
                 'bias=' + str(self.bias is not None)).format(**self.__dict__)
 
 
+class _ConvOffsetPackNd(_ConvOffsetNd):
+    """The deformable layer together with its offset-producing convolution (MIOpen through
+    `nn.Conv{2,3}d`).  The offset convolution uses the layer's kernel size, stride and padding
+    with dilation 1: its output then has the layer's (dilation-blind) output size for every
+    dilation, which the callers' own construction only achieves for dilation 1.
+    `zero_init_offset=True` starts from zero offsets (the layer then equals a plain convolution
+    sampled at the integer taps); the default keeps PyTorch's initialisation, as the reference's
+    callers do.  Parameters: `weight`, `bias` (as ConvOffsetNd) and `conv_offset.weight`."""
+    _conv = None
+    _nd = None
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 channel_per_group=1, bias=True, groups=1, zero_init_offset=False, device=None, dtype=None):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, channel_per_group,
+                         bias, groups, device=device, dtype=dtype)
+        if in_channels % channel_per_group != 0:
+            raise ValueError('in_channels must be divisible by channel_per_group')
+        taps = 1
+        for k in self.kernel_size:
+            taps *= k
+        self.conv_offset = self._conv(in_channels, in_channels // channel_per_group * self._nd * taps,
+                                      self.kernel_size, self.stride, self.padding, bias=False,
+                                      device=device, dtype=dtype)
+        if zero_init_offset:
+            nn.init.zeros_(self.conv_offset.weight)
+
+    def forward(self, input):
+        return super().forward(input, self.conv_offset(input))
+
+
 class ConvOffset3d(_ConvOffsetNd):
     _tuple = staticmethod(_triple)
     _function = ConvOffset3dFunction
@@ -67,3 +102,17 @@ class ConvOffset3d(_ConvOffsetNd):
 class ConvOffset2d(_ConvOffsetNd):
     _tuple = staticmethod(_pair)
     _function = ConvOffset2dFunction
+
+
+class ConvOffset3dPack(_ConvOffsetPackNd):
+    _tuple = staticmethod(_triple)
+    _function = ConvOffset3dFunction
+    _conv = nn.Conv3d
+    _nd = 3
+
+
+class ConvOffset2dPack(_ConvOffsetPackNd):
+    _tuple = staticmethod(_pair)
+    _function = ConvOffset2dFunction
+    _conv = nn.Conv2d
+    _nd = 2

@@ -166,6 +166,60 @@ def test_modules_forward_backward():
     assert sorted(m3.state_dict()) == ["bias", "weight"]
 
 
+class _OracleLayer(torch.autograd.Function):
+    """The CPU oracle as an autograd node, so that a CPU graph (offset convolution -> layer) can be
+    differentiated end to end as the reference for the Pack modules."""
+
+    @staticmethod
+    def forward(ctx, x, off, w, b, cfg):
+        ctx.save_for_backward(x, off, w, b)
+        ctx.cfg = cfg
+        return orc.forward(x.detach(), off.detach(), w.detach(), b.detach(), *cfg)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, off, w, b = ctx.saved_tensors
+        gin, goff, gw, gb = orc.backward(x.detach(), off.detach(), w.detach(), g.contiguous(), b.detach(), *ctx.cfg)
+        return gin, goff, gw, gb, None
+
+
+@pytest.mark.parametrize("nd", [2, 3])
+def test_pack_module_end_to_end(nd):
+    """ConvOffset{2,3}dPack (offset convolution + layer) against the same graph on the CPU: torch's
+    convolution for the offsets, the oracle for the layer; float64, all four gradients."""
+    print("pack module", nd, flush=True)
+    dcn = _dcn()
+    dev = "cuda:0"
+    torch.manual_seed(3)
+    if nd == 3:
+        m = dcn.ConvOffset3dPack(6, 4, 3, stride=(1, 2, 1), padding=1, dilation=(1, 1, 2), channel_per_group=3, groups=2,
+                                 dtype=torch.float64)
+        x = torch.randn(2, 6, 4, 7, 6, dtype=torch.float64)
+    else:
+        m = dcn.ConvOffset2dPack(4, 6, (3, 2), stride=1, padding=(1, 0), dilation=1, channel_per_group=2, groups=2,
+                                 dtype=torch.float64)
+        x = torch.randn(2, 4, 7, 6, dtype=torch.float64)
+    with torch.no_grad():
+        m.conv_offset.weight.mul_(4.0)                 # offsets of a few voxels, some samples out of range
+    ref = {k: v.detach().clone().requires_grad_(True) for k, v in m.named_parameters()}
+    xr = x.clone().requires_grad_(True)
+    conv = torch.nn.functional.conv3d if nd == 3 else torch.nn.functional.conv2d
+    off_r = conv(xr, ref["conv_offset.weight"], None, m.stride, m.padding)
+    cfg = (m.stride, m.padding, m.dilation, m.channel_per_group, m.group)
+    out_r = _OracleLayer.apply(xr, off_r, ref["weight"], ref["bias"], cfg)
+    gout = torch.randn_like(out_r)
+    out_r.backward(gout)
+
+    m = m.to(dev)
+    xg = x.to(dev).requires_grad_(True)
+    out = m(xg)
+    out.backward(gout.to(dev))
+    assert rel_err(out, out_r) < 1e-10
+    assert rel_err(xg.grad, xr.grad) < 1e-10
+    for k, v in m.named_parameters():
+        assert rel_err(v.grad, ref[k].grad) < 1e-10, k
+
+
 def test_needs_input_grad_gating():
     dcn = _dcn()
     dev = "cuda:0"

@@ -125,3 +125,21 @@ def test_reference_function_script_values():
     assert out[1, 0, 1] == 8.0
     # zero offsets at integer coordinates: grad_offset is the finite difference toward the high corner
     assert d["gw"].shape == (1, 1, 3, 3, 3)
+
+
+def test_pack_modules_construction():
+    """The modules that own the offset convolution: parameter names, offset channels, offset size."""
+    import deform_conv3d_pytorch_op_amd as dcn
+    m = dcn.ConvOffset3dPack(8, 6, (3, 3, 1), stride=(1, 2, 1), padding=(1, 1, 0), dilation=2, channel_per_group=4, groups=2)
+    assert sorted(m.state_dict()) == ["bias", "conv_offset.weight", "weight"]
+    assert tuple(m.conv_offset.weight.shape) == (8 // 4 * 3 * 9, 8, 3, 3, 1)
+    x = torch.randn(2, 8, 5, 8, 4)
+    # the offset convolution (dilation 1) has the layer's dilation-blind output size
+    assert tuple(m.conv_offset(x).shape[2:]) == dcn.output_size((5, 8, 4), (3, 3, 1), (1, 2, 1), (1, 1, 0))
+    m2 = dcn.ConvOffset2dPack(4, 4, 3, padding=1, channel_per_group=2, bias=False, zero_init_offset=True)
+    assert sorted(m2.state_dict()) == ["conv_offset.weight", "weight"]
+    assert float(m2.conv_offset.weight.abs().max()) == 0.0
+    with pytest.raises(ValueError):
+        dcn.ConvOffset2dPack(6, 4, 3, channel_per_group=4)
+    with pytest.raises(RuntimeError):          # no CPU path: the layer itself needs the GPU
+        m2(torch.randn(1, 4, 5, 5))
