@@ -30,8 +30,8 @@ template <typename T> void fwd_weight_pad(int M, int Cg, int& MT, int& mchunks, 
     Mp = mchunks * MT * TN;
     Cgp = Cg + 2 * KL;       // the kernels read up to one reduction step past the last channel
 }
-// backward-data layout.  MK = reduction steps over output channels kept in registers by
-// backward_input_halo_kernel (0: M too large, the kernel re-reads grad_output per tap).
+// backward-data layout.  MK = reduction steps over output channels whose grad_output values
+// backward_data_kernel keeps in registers (0: M too large, the kernel re-reads grad_output per tap).
 template <typename T> int bwd_data_mk(int M) {
     const int steps = (M + Mma<T>::KL - 1) / Mma<T>::KL;
     for (int mk = 8; mk <= 64; mk *= 2)

@@ -708,13 +708,15 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // Same halo tiling as forward_halo_kernel, but the LDS planes hold the partial grad-input of CCH
 // channels over the halo of the workgroup's position block (cells: see LdsCell).  The rows of
 // one MFMA tile are (tap, channel) pairs -- TP = TN / CCH taps of the CCH channels -- so a pass
-// of MK MFMAs yields the grad-column values gcol[c][tap][pos] of TP taps at once with lanes
-// along positions.  Each lane then walks its registers: per tap it derives the corner indices
-// and weights of its position and adds (w_l*w_h*w_w)*gcol to the 8 (4) corners with LDS integer
-// atomics.  After all taps the planes are added to grad_input with one hardware float atomic per
-// touched halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that
-// reach past the halo use global atomics directly.
-// dynamic LDS = CCH * hstride * 8 + hvol * 4 + kV * ND * 4 bytes.
+// of ceil(M / KL) MFMAs yields the grad-column values gcol[c][tap][pos] of TP taps at once with
+// lanes along positions.  Each lane then walks its registers: per tap slot it derives the corner
+// cells and weights of its position once, per channel it adds (w_l*w_h*w_w)*gcol to the 8 (4)
+// corners with LDS integer atomics.  The MFMAs of the next pass are issued between those steps.
+// After all taps the planes are added to grad_input with one hardware float atomic per touched
+// halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that reach past
+// the halo use global atomics directly, in a pass of their own.
+// 1-D grid of DG * N * tiles * csplit workgroups; dynamic LDS = CCH * hstride * 8 + hvol * 4 +
+// kV * ND * 4 bytes.
 // COORD = true additionally stages the same CCH input channels over the halo (float planes) and
 // computes grad_offset in the same pass over the grad-column values (col2im_offset of the
 // reference, deform3d kernel.cu:386-483 incl. the out-of-range branches :470-481, 2-D
