@@ -448,7 +448,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
 
 // Plan of backward_weight: channel tiles, m chunks and the number of position splits.
 template <typename T>
-void bww_plan(const Params& Pin, int& MT, int& mchunks, int& nct, int& nsplit) {
+void bww_plan(const Params& Pin, int& MT, int& mchunks, int& nct, int& nsplit, long long resident = 0) {
     const int TN = Mma<T>::TN;
     const int mtiles = (Pin.M + TN - 1) / TN;
     MT = mtiles > 2 ? 4 : mtiles;
@@ -463,15 +463,36 @@ void bww_plan(const Params& Pin, int& MT, int& mchunks, int& nct, int& nsplit) {
             nct += (ce - cb + TN - 1) / TN;
         }
     }
-    // split the position reduction so that the grid holds a few thousand workgroups
+    // split the position reduction so that the grid holds a few thousand workgroups: the largest
+    // whole number of rounds of resident workgroups below about 4096 (a grid just past a whole
+    // number of rounds pays a full round for the remainder)
     const long long slabs = (long long)Pin.N * ((Pin.outV + TN - 1) / TN);
     const long long other = (long long)Pin.kV * nct * mchunks;
     long long split = (4096 + other - 1) / other;
+    if (resident > 0 && resident <= 4096) {
+        const long long balanced = (4096 / resident) * resident / other;
+        if (balanced >= 1 && balanced < split) split = balanced;
+    }
     const long long max_split = (slabs + WAVES - 1) / WAVES;
     if (split > max_split) split = max_split;
     if (split > 256) split = 256;
     if (split < 1) split = 1;
     nsplit = (int)split;
+}
+
+// Workgroups of backward_weight_kernel that the device holds at once (0 if the query fails).
+template <typename T, int ND, int MT>
+long long bww_resident() {
+    static const long long v = [] {
+        int per_cu = 0;
+        const size_t lds = (size_t)WAVES * Mma<T>::TN * (Mma<T>::TN + 1) * sizeof(T);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, backward_weight_kernel<T, ND, MT>, WG, lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0LL;
+        }
+        return (long long)per_cu * cu_count();
+    }();
+    return v;
 }
 
 template <typename T, int ND, int MT>
@@ -506,6 +527,8 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     if ((long long)P.outV * P.C_out > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one output sample exceeds 2^31 elements");
     int MT;
     bww_plan<T>(P, MT, P.mchunks, P.nctiles, P.nsplit);
+    const long long resident = MT == 1 ? bww_resident<T, ND, 1>() : MT == 2 ? bww_resident<T, ND, 2>() : bww_resident<T, ND, 4>();
+    bww_plan<T>(P, MT, P.mchunks, P.nctiles, P.nsplit, resident);
     if ((long long)P.nctiles * P.mchunks > 65535) return fail(DCN_E_ARGUMENT, "too many channel tiles for one launch");
     const size_t ibytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
     const size_t obytes = align256((size_t)P.N * P.C_out * P.outV * sizeof(T));
