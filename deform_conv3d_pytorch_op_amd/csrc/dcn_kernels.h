@@ -904,6 +904,26 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 for (int a = 0; a < ND; ++a) kd_nx[a] = sKd[(tu + dqc) * ND + a];
             };
             load_slot_offsets(MM::row(0, 0) / CCH, 0);
+            // grad_offset of a finished tap slot, held back until the loads of the next slot have been
+            // issued: vector memory operations complete in order, so a load issued behind these
+            // stores / atomics could only be waited for together with them
+            bool pend = false;
+            int pend_tap = 0;
+            T pend_ga[ND];
+#pragma unroll
+            for (int a = 0; a < ND; ++a) pend_ga[a] = 0;
+            auto write_goff = [&]() {
+                if (pend) {
+                    T* gp = goff_dg + (size_t)pend_tap * ND * P.outV + pos;
+#pragma unroll
+                    for (int a = 0; a < ND; ++a) {
+                        if (csplit > 1) { if (pend_ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, pend_ga[a]); }
+                        else if (first_chunk) gp[(size_t)a * P.outV] = pend_ga[a];
+                        else gp[(size_t)a * P.outV] += pend_ga[a];
+                    }
+                }
+                pend = false;
+            };
 
             for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
                 const typename MM::Acc d = d_next;
@@ -928,6 +948,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     if (do_mma) load_batch(a_cu, b_cu, wnext, ts * AB);
                     if (ts + 1 < NS) load_slot_offsets(tap0 + MM::row((ts + 1) * RPS, 0) / CCH, ts + 1);
                     else load_slot_offsets(tap0 + TP + MM::row(0, 0) / CCH, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (COORD) write_goff();
                     __builtin_amdgcn_sched_barrier(0);
 
                     TapGeo<T, ND> t;
@@ -1042,20 +1064,17 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                                 for (int sh = TN; sh < TN * (CCH / RPS); sh <<= 1) ga[a] += __shfl_xor(ga[a], sh);
                         }
+                        // written at the start of the next slot, behind that slot's loads (see write_goff)
                         const bool owner = (RPS == CCH) || (q % (CCH / RPS)) == 0;
-                        if (slot_ok && owner) {
-                            T* gp = goff_dg + (size_t)tap * ND * P.outV + pos;
+                        pend = slot_ok && owner;
+                        pend_tap = tap;
 #pragma unroll
-                            for (int a = 0; a < ND; ++a) {
-                                if (csplit > 1) { if (ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, ga[a]); }
-                                else if (first_chunk) gp[(size_t)a * P.outV] = ga[a];
-                                else gp[(size_t)a * P.outV] += ga[a];
-                            }
-                        }
+                        for (int a = 0; a < ND; ++a) pend_ga[a] = ga[a];
                     }
                     __builtin_amdgcn_sched_barrier(0);      // one tap slot at a time: keeps the live register set small
                 }
             }
+            if constexpr (COORD) write_goff();
             first_chunk = false;
             __syncthreads();                        // all LDS adds of this chunk have landed
             for (int v = threadIdx.x; v < P.hvol; v += WGS) {
