@@ -166,6 +166,24 @@ def test_modules_forward_backward():
     assert sorted(m3.state_dict()) == ["bias", "weight"]
 
 
+@pytest.mark.parametrize("name", ["3d_basic", "2d_basic", "3d_c5_like"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+def test_non_finite_and_huge_offsets(name, dtype):
+    """Offsets that are NaN, infinite or far beyond the integer range select no voxel (every window
+    test of the sampler is false for them): those samples add nothing, on the GPU as in the oracle."""
+    print("special offsets", name, dtype, flush=True)
+    c = make_case(*SMALL_CASES[name], dtype=dtype, seed=5)
+    flat = c["off"].view(-1)
+    idx = torch.randperm(flat.numel(), generator=torch.Generator().manual_seed(1))[:64]
+    vals = torch.tensor([float("nan"), float("inf"), -float("inf"), 1e30, -1e30, 3e9, -3e9, 1e5], dtype=dtype)
+    flat[idx] = vals[torch.arange(64) % 8]
+    got = run_gpu(c)
+    want = run_oracle(c)
+    for nm, g, w in zip(("output", "grad_input", "grad_offset", "grad_weight", "grad_bias"), got, want):
+        assert torch.isfinite(g).all(), nm
+        assert rel_err(g, w) < TOL[dtype]["fwd" if nm == "output" else "grad"], nm
+
+
 class _OracleLayer(torch.autograd.Function):
     """The CPU oracle as an autograd node, so that a CPU graph (offset convolution -> layer) can be
     differentiated end to end as the reference for the Pack modules."""
