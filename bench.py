@@ -74,8 +74,8 @@ def algorithmic_bytes(c):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c4", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -129,6 +129,20 @@ def main():
         fwd_only()
     torch.cuda.synchronize()
     ms_fwd = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    # the same two quantities step by step between HIP events (median and minimum), outside the timed region above
+    def event_times(fn_):
+        evs = []
+        for _ in range(a.steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn_()
+            e1.record()
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        ts = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+        return {"median": round(ts[len(ts) // 2], 4), "min": round(ts[0], 4)}
+    step_events, fwd_events = event_times(step), event_times(fwd_only)
 
     F = gemm_flops(c)
     value = 3 * F / (ms_step * 1e-3) / 1e12
@@ -209,7 +223,8 @@ def main():
     print(json.dumps({
         "metric": "deform conv fwd+bwd effective TFLOP/s per layer (3 dense contractions counted)",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(ms_step, 4), "fwd_ms": round(ms_fwd, 4), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": round(ms_step, 4), "fwd_ms": round(ms_fwd, 4),
+        "ms_per_step_events": step_events, "fwd_ms_events": fwd_events, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32" if dtype == torch.float32 else "f64", "data": "synthetic",
         "config": {"workload": a.config + ": " + DESCR[a.config]},
         "mfma_frac_whole_step": round(value / peak, 4),
