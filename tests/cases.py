@@ -53,5 +53,8 @@ SMALL_CASES = {
     "3d_c4_like": (3, 2, 40, 40, (4, 9, 10), 3, 1, 1, 1, 40, 1, 1.5),      # one deformable group, >1 channel tile
     "3d_c5_like": (3, 1, 16, 24, (4, 12, 12), 3, (1, 2, 2), 1, 1, 4, 1, 2.0),   # strided, 4 deformable groups
     "3d_wide_m": (3, 1, 8, 136, (3, 6, 6), 3, 1, 1, 1, 8, 1, 2.0),        # more reduction steps than one pass of tap slots takes
+    "2d_k5_depthwise": (2, 1, 6, 6, (9, 9), 5, 1, 2, 1, 1, 6, 1.0),         # 25 taps, one channel per group and per deformable group
+    "3d_k1_stride3": (3, 2, 5, 7, (5, 7, 6), 1, 3, 0, 1, 5, 1, 2.0),         # a single tap, odd channel counts, stride > kernel
+    "3d_dilation3": (3, 1, 4, 4, (8, 8, 8), 3, 1, 3, 3, 2, 1, 2.5),          # dilation-blind output 12^3: many taps out of range
     "3d_short_length": (3, 1, 4, 4, (2, 8, 8), (1, 3, 3), 1, (0, 1, 1), 1, 4, 1, 4.0),  # D < H: out-of-range branch vs length extent
 }
