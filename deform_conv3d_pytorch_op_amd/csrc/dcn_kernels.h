@@ -854,9 +854,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             // used instead of being hoisted out of the loops into hundreds of long-lived registers)
             auto load_batch = [&](T* a_nx, T* b_nx, const T* wp, int k0) {      // rows past M are zero padding
                 asm volatile("" : "+s"(k0));
+                const T* wb = wp + (size_t)k0 * wstep;                 // one 64-bit product per batch; the row offsets below are loop invariants
 #pragma unroll
                 for (int k = 0; k < AB; ++k) {
-                    a_nx[k] = (wp + (size_t)(k0 + k) * wstep)[a_off];
+                    a_nx[k] = (wb + (unsigned)k * (unsigned)wstep)[a_off];
                     if constexpr (!BREG) b_nx[k] = load_b(k0 + k, false);
                 }
             };
