@@ -207,8 +207,8 @@ def main():
         from oracle import dcn_oracle as orc
         ns = x.shape[0]
         xs, offs, gs = c["x"][:ns].contiguous(), c["off"][:ns].contiguous(), c["gout"][:ns].contiguous()
-        reps, times = (5 if a.config in ("c4", "c5") else 9), []
-        for _ in range(reps):                  # about 5-10 s of host work at c4
+        reps, times = 9, []
+        for _ in range(reps):                  # about 12 s of host work at c4 (16 threads)
             t0 = time.perf_counter()
             orc.forward(xs, offs, c["w"], None, *cfg, acc64=False)
             orc.backward(xs, offs, c["w"], gs, None, *cfg, acc64=False)
