@@ -238,6 +238,18 @@ def test_pack_module_end_to_end(nd):
         assert rel_err(v.grad, ref[k].grad) < 1e-10, k
 
 
+def test_forward_and_grad_weight_are_deterministic():
+    """No float atomics on these two paths: repeated calls give identical bits.  (grad_input and
+    grad_offset end in float atomics and may differ in the last bits from run to run.)"""
+    c = make_case(*SMALL_CASES["3d_c4_like"], dtype=torch.float32, seed=4)
+    first = run_gpu(c)
+    for _ in range(3):
+        again = run_gpu(c)
+        assert torch.equal(first[0], again[0])
+        assert torch.equal(first[3], again[3])
+        assert rel_err(again[1], first[1].cpu()) < 1e-5 and rel_err(again[2], first[2].cpu()) < 1e-5
+
+
 def test_hip_graph_replay():
     """Forward + backward captured into a HIP graph (the C ABI allocates nothing, clears memory with
     kernels only and never synchronises); every replay, with eager work and synchronisations in
