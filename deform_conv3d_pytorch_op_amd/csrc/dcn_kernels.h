@@ -223,6 +223,23 @@ __device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, 
     }
 }
 
+// The same for a channel-interleaved halo [halo voxel][CCH]: the CCH channel values of a voxel sit
+// next to each other, so one wide LDS read fetches a corner of all of them (missing channels of a
+// short last chunk are stored as zero).
+template <typename T, int CCH, int WGS>
+__device__ inline void halo_stage_interleaved(const Params& P, const T* __restrict__ chan0, int nch,
+                                              const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
+    for (int v = threadIdx.x; v < P.hvol; v += WGS) {
+        const unsigned t = sTab[v];
+        const unsigned g = t == ~0u ? 0u : t;
+        T val[CCH];
+#pragma unroll
+        for (int c = 0; c < CCH; ++c) val[c] = chan0[(size_t)min(c, nch - 1) * P.inV + g];   // CCH loads in flight
+#pragma unroll
+        for (int c = 0; c < CCH; ++c) sIn[(size_t)v * CCH + c] = c < nch ? val[c] : (T)0;
+    }
+}
+
 // LDS indices of the corners of an inside sample; false if any corner lies outside the halo
 template <typename T, int ND>
 __device__ inline bool halo_corners(const Params& P, const int hb[ND], const TapGeo<T, ND>& t, unsigned lidx[1 << ND]) {
@@ -745,7 +762,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int hs = HS ? HS : P.hstride;
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
-    T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * hs);                               // [CCH][hstride] if COORD
+    T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * hs);                               // [hstride][CCH] if COORD: channels of a voxel side by side
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
     int* sKd = reinterpret_cast<int*>(sTab + P.hvol);                                   // [kV][ND]: tap * dilation per axis
     constexpr int WGS = NW * 64;                        // threads per workgroup
@@ -837,7 +854,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
                 for (int v = threadIdx.x; v < P.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
-            if constexpr (COORD) halo_stage<T, WGS>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
+            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
 
             // Grad-column tile of a pass: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past
@@ -987,24 +1004,48 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     Cell* g_cell[NC];
                     const T* in_cell[NC];
 #pragma unroll
-                    for (int i = 0; i < NC; ++i) { g_cell[i] = sG + lidx[i]; in_cell[i] = sIn + lidx[i]; }
-                    // d(sample)/d(coordinate) of one channel from its corner values, times gcol
-                    // (the w-lerps of the four (l, h) corner pairs are shared by the l and h derivatives)
-                    auto coord_grad = [&](const T v[NC], T gv) {
+                    for (int i = 0; i < NC; ++i) { g_cell[i] = sG + lidx[i]; in_cell[i] = sIn + (size_t)lidx[i] * CCH; }
+                    // d(sample)/d(coordinate) from corner values; the formula is linear in them, so it is
+                    // applied once per tap slot to the corner values weighted by gcol and summed over the
+                    // lane's channels (the w-lerps of the four (l, h) corner pairs are shared by the l
+                    // and h derivatives)
+                    auto coord_grad = [&](const T v[NC]) {
                         if constexpr (ND == 3) {
                             const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
                             const T c00 = v[0] * gw + v[1] * fw, c01 = v[2] * gw + v[3] * fw;
                             const T c10 = v[4] * gw + v[5] * fw, c11 = v[6] * gw + v[7] * fw;
-                            ga[0] += gv * ((c10 - c00) * gh + (c11 - c01) * fh);
-                            ga[1] += gv * ((c01 - c00) * gl + (c11 - c10) * fl);
-                            ga[2] += gv * (((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
-                                           ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl);
+                            ga[0] += (c10 - c00) * gh + (c11 - c01) * fh;
+                            ga[1] += (c01 - c00) * gl + (c11 - c10) * fl;
+                            ga[2] += ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                     ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
                         } else {
                             const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                            ga[0] += gv * ((v[2] - v[0]) * gw + (v[3] - v[1]) * fw);
-                            ga[1] += gv * ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh);
+                            ga[0] += (v[2] - v[0]) * gw + (v[3] - v[1]) * fw;
+                            ga[1] += (v[1] - v[0]) * gh + (v[3] - v[2]) * fh;
                         }
                     };
+                    // corner values of the input, one wide LDS read per corner for all of this lane's
+                    // channels, weighted by their grad-column values.  The reads go first: LDS operations
+                    // complete in order, so this waits for them only, not for the adds issued below
+                    T gsum[NC];
+                    if constexpr (COORD) {
+                        if (near) {
+                            T gvc[RPS];
+#pragma unroll
+                            for (int rr = 0; rr < RPS; ++rr)
+                                gvc[rr] = (MM::row(ts * RPS + rr, q) % CCH) < nch ? d[ts * RPS + rr] : (T)0;
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) {
+                                T vv[RPS];
+#pragma unroll
+                                for (int rr = 0; rr < RPS; ++rr) vv[rr] = in_cell[i][MM::row(ts * RPS + rr, q) % CCH];
+                                T acc_ = 0;
+#pragma unroll
+                                for (int rr = 0; rr < RPS; ++rr) acc_ += gvc[rr] * vv[rr];
+                                gsum[i] = acc_;
+                            }
+                        }
+                    }
 #pragma unroll
                     for (int rr = 0; rr < RPS; ++rr) {
                         const int r = ts * RPS + rr;
@@ -1012,17 +1053,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         const T gv = d[r];
                         if (cl >= nch) {
                         } else if (near) {
-                            // the reads go first: LDS operations complete in order, so the interpolation
-                            // gradient below waits for them only, not for the adds issued after them
-                            T v[NC];
-                            if constexpr (COORD) {
-#pragma unroll
-                                for (int i = 0; i < NC; ++i) v[i] = in_cell[i][cl * hs];
-                            }
                             const double gs = LdsCell<T>::pre(gv, scale);
 #pragma unroll
                             for (int i = 0; i < NC; ++i) LdsCell<T>::add(g_cell[i] + cl * hs, cwd[i], gs);
-                            if constexpr (COORD) coord_grad(v, gv);
                         } else if (oor) {
                             const T av = gv > 0 ? gv : -gv;
 #pragma unroll
@@ -1034,6 +1067,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                             for (int k = 0; k < MPR; ++k)
                                 d_next = MM::mma(a_cu[rr * MPR + k], BREG ? b_reg[ts * AB + rr * MPR + k] : b_cu[rr * MPR + k], d_next);
                         }
+                    }
+                    if constexpr (COORD) {
+                        if (near) coord_grad(gsum);
                     }
                     if (__any(far)) {              // rare: samples that reach past the halo go to global memory
                         tap_corner_idx<T, ND>(P, t);
@@ -1051,8 +1087,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                                     const T* ic = in + chan;
                                     T v[NC];
 #pragma unroll
-                                    for (int i = 0; i < NC; ++i) v[i] = ic[t.idx[i]];
-                                    coord_grad(v, gv);
+                                    for (int i = 0; i < NC; ++i) v[i] = gv * ic[t.idx[i]];
+                                    coord_grad(v);
                                 }
                             }
                         }
