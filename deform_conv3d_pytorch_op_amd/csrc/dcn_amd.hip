@@ -91,7 +91,12 @@ int validate(const Geometry& g, Params& P) {
         if (g.in[a] <= 0 || g.k[a] <= 0 || g.stride[a] <= 0 || g.dil[a] <= 0 || g.pad[a] < 0)
             return fail(DCN_E_ARGUMENT, "input / kernel / stride / dilation extents must be positive, pad non-negative");
         if (g.in[a] + 2 * g.pad[a] - g.k[a] < 0) return fail(DCN_E_ARGUMENT, omsg[a]);
-        if ((g.in[a] + 2 * g.pad[a] - g.k[a]) / g.stride[a] + 1 != g.out[a]) return fail(DCN_E_ARGUMENT, omsg[a]);
+        // the reference's dilation-blind output size, or the usual dilation-aware one (the sampler
+        // gives every position a meaning, so both are served)
+        const int blind = (g.in[a] + 2 * g.pad[a] - g.k[a]) / g.stride[a] + 1;
+        const int span = g.in[a] + 2 * g.pad[a] - g.dil[a] * (g.k[a] - 1) - 1;
+        const int standard = span >= 0 ? span / g.stride[a] + 1 : 0;
+        if (g.out[a] != blind && !(standard >= 1 && g.out[a] == standard)) return fail(DCN_E_ARGUMENT, omsg[a]);
     }
     const long long inV = (long long)g.in[0] * g.in[1] * g.in[2], outV = (long long)g.out[0] * g.out[1] * g.out[2];
     // per-channel offsets are 32-bit inside the kernels (including a bias of up to 4 channels)

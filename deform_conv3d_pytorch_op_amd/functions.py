@@ -5,7 +5,8 @@ deform2d/deform_conv2d_functions/deform_conv2d_function.py:7-57 is its float, di
 group-1, bias-free subset).
 
 Same call shape: `Fn.apply(inputs, offset, weight, bias=None, stride, padding, dilation,
-channel_per_group=1, group=1)`; same dilation-blind output size; same shape checks and messages
+channel_per_group=1, group=1)` (plus one optional trailing argument, `standard_output_size`, see
+`output_size`); same dilation-blind output size by default; same shape checks and messages
 as the reference's `shape_check` (deform3d/lib/deform_conv3d_cuda.cpp:24-87), raised as
 RuntimeError.  Differences: no column workspace is kept on ctx (the kernels never build one),
 float32 and float64 are served by the same class for both 2-D and 3-D, and gradients that are
@@ -34,9 +35,16 @@ def _ntuple(v, nd):
     return v
 
 
-def output_size(in_sizes, kernel, stride, padding):
+def output_size(in_sizes, kernel, stride, padding, dilation=None, standard=False):
     """The reference formula, dilation not included (deform3d/lib/deform_conv3d_cuda.cpp:15-17;
-    deform_conv3d_function.py:26-27)."""
+    deform_conv3d_function.py:26-27).  `standard=True` gives the usual dilation-aware size
+    `(in + 2p - d(k-1) - 1) // s + 1` instead (the one the reference's plain convolution uses,
+    conv2d/lib/conv2d_cuda.cpp:20-22): with it every tap of every output position starts inside
+    the padded input, as in an ordinary convolution."""
+    if standard:
+        dilation = dilation if dilation is not None else (1,) * len(kernel)
+        return tuple((i + 2 * p - d * (k - 1) - 1) // s + 1
+                     for i, k, s, p, d in zip(in_sizes, kernel, stride, padding, dilation))
     return tuple((i + 2 * p - k) // s + 1 for i, k, s, p in zip(in_sizes, kernel, stride, padding))
 
 
@@ -44,7 +52,8 @@ _OUT_MSG = {3: ("error output ll", "error outhh", "error outww"), 2: ("error out
 _OFF_MSG = {3: ("off l", "off h", "off w"), 2: ("off h", "off w")}
 
 
-def shape_check(nd, inputs, weight, offset, output_shape, channel_per_group, group, stride, padding):
+def shape_check(nd, inputs, weight, offset, output_shape, channel_per_group, group, stride, padding,
+                dilation=None, standard=False):
     """Python restatement of the reference's shape_check with its messages."""
     _check(weight.dim() == nd + 2, "kernel dim")
     _check(inputs.dim() == nd + 2, "input dim")
@@ -61,10 +70,10 @@ def shape_check(nd, inputs, weight, offset, output_shape, channel_per_group, gro
     _check(offset.size(1) == inputs.size(1) // channel_per_group * nd * kV, "off channel")
     for a in range(nd):
         _check(offset.size(2 + a) == output_shape[2 + a], _OFF_MSG[nd][a])
-    want = output_size(inputs.shape[2:], weight.shape[2:], stride, padding)
+    want = output_size(inputs.shape[2:], weight.shape[2:], stride, padding, dilation, standard)
     for a in range(nd):
-        _check(inputs.size(2 + a) + 2 * padding[a] - weight.size(2 + a) >= 0 and want[a] == output_shape[2 + a],
-               _OUT_MSG[nd][a])
+        _check(inputs.size(2 + a) + 2 * padding[a] - weight.size(2 + a) >= 0 and want[a] >= 1 and
+               want[a] == output_shape[2 + a], _OUT_MSG[nd][a])
     _check(group > 0 and weight.size(0) % group == 0, "ou c != ker c")
 
 
@@ -103,15 +112,15 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group):
+def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group, standard=False):
     L = _lib.load()
     stride, padding, dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
     _device_check(inputs, offset, weight, bias)
     _check(inputs.dim() == nd + 2, "input dim")
     _check(weight.dim() == nd + 2, "kernel dim")
-    outs = output_size(inputs.shape[2:], weight.shape[2:], stride, padding)
+    outs = output_size(inputs.shape[2:], weight.shape[2:], stride, padding, dilation, standard)
     out_shape = (inputs.size(0), weight.size(0)) + outs
-    shape_check(nd, inputs, weight, offset, out_shape, channel_per_group, group, stride, padding)
+    shape_check(nd, inputs, weight, offset, out_shape, channel_per_group, group, stride, padding, dilation, standard)
     if bias is not None:
         _check(bias.dim() == 1 and bias.size(0) == weight.size(0), "bias size")
     inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
@@ -128,11 +137,12 @@ def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channe
 
 
 def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation, channel_per_group, group,
-              need_data, need_weight):
+              need_data, need_weight, standard=False):
     L = _lib.load()
     _device_check(inputs, offset, weight, grad_output)
     outs = tuple(grad_output.shape[2:])
-    shape_check(nd, inputs, weight, offset, tuple(grad_output.shape), channel_per_group, group, stride, padding)
+    shape_check(nd, inputs, weight, offset, tuple(grad_output.shape), channel_per_group, group, stride, padding,
+                dilation, standard)
     inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
     grad_output = grad_output.contiguous()
     geom = _geom(nd, inputs, weight, outs, stride, padding, dilation, channel_per_group, group)
@@ -160,14 +170,16 @@ class _ConvOffsetNdFunction(Function):
     ND = 0
 
     @classmethod
-    def _fwd(cls, ctx, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group):
+    def _fwd(cls, ctx, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group,
+             standard_output_size=False):
         nd = cls.ND
+        ctx.standard = bool(standard_output_size)
         ctx.stride, ctx.padding, ctx.dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
         ctx.channel_per_group, ctx.group = int(channel_per_group), int(group)
         ctx.has_bias = bias is not None
         ctx.save_for_backward(inputs, offset, weight)
         return _forward(nd, inputs, offset, weight, bias, ctx.stride, ctx.padding, ctx.dilation,
-                        ctx.channel_per_group, ctx.group)
+                        ctx.channel_per_group, ctx.group, ctx.standard)
 
     @classmethod
     def _bwd(cls, ctx, grad_output):
@@ -175,11 +187,11 @@ class _ConvOffsetNdFunction(Function):
         need = ctx.needs_input_grad
         # grad_input and grad_offset come out of one kernel, as in the reference (:52)
         gi, go, gw = _backward(cls.ND, inputs, offset, weight, grad_output, ctx.stride, ctx.padding, ctx.dilation,
-                               ctx.channel_per_group, ctx.group, need[0] or need[1], need[2])
+                               ctx.channel_per_group, ctx.group, need[0] or need[1], need[2], ctx.standard)
         gb = None
         if ctx.has_bias and need[3]:
             gb = grad_output.sum(dim=[0] + list(range(2, 2 + cls.ND)))
-        return (gi if need[0] else None, go if need[1] else None, gw, gb, None, None, None, None, None)
+        return (gi if need[0] else None, go if need[1] else None, gw, gb, None, None, None, None, None, None)
 
 
 class ConvOffset3dFunction(_ConvOffsetNdFunction):
@@ -187,9 +199,9 @@ class ConvOffset3dFunction(_ConvOffsetNdFunction):
 
     @staticmethod
     def forward(ctx, inputs, offset, weight, bias=None, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
-                channel_per_group=1, group=1):
+                channel_per_group=1, group=1, standard_output_size=False):
         return ConvOffset3dFunction._fwd(ctx, inputs, offset, weight, bias, stride, padding, dilation,
-                                         channel_per_group, group)
+                                         channel_per_group, group, standard_output_size)
 
     @staticmethod
     @once_differentiable
@@ -202,9 +214,9 @@ class ConvOffset2dFunction(_ConvOffsetNdFunction):
 
     @staticmethod
     def forward(ctx, inputs, offset, weight, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
-                channel_per_group=1, group=1):
+                channel_per_group=1, group=1, standard_output_size=False):
         return ConvOffset2dFunction._fwd(ctx, inputs, offset, weight, bias, stride, padding, dilation,
-                                         channel_per_group, group)
+                                         channel_per_group, group, standard_output_size)
 
     @staticmethod
     @once_differentiable

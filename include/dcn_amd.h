@@ -38,6 +38,9 @@
  * a plain gradient is wanted (deform3d/deform_conv3d_functions/deform_conv3d_function.py:53,64).
  * Output extents must satisfy the reference formula out = (in + 2*pad - kernel) / stride + 1
  * (integer division, dilation not included; deform3d/lib/deform_conv3d_cuda.cpp:15-17,81-86).
+ * The dilation-aware size (in + 2*pad - dilation*(kernel-1) - 1) / stride + 1 is accepted as
+ * well: it is the same layer cropped to the leading positions of each axis (no counterpart in
+ * the reference, which always uses the first formula).
  */
 #ifndef DCN_AMD_H
 #define DCN_AMD_H

@@ -184,6 +184,66 @@ def test_non_finite_and_huge_offsets(name, dtype):
         assert rel_err(g, w) < TOL[dtype]["fwd" if nm == "output" else "grad"], nm
 
 
+@pytest.mark.parametrize("name", ["2d_c3_like", "2d_rect_kernel_stride_dil", "3d_dilation3", "3d_basic"])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32], ids=["f64", "f32"])
+def test_standard_output_size_is_a_crop_of_the_reference_layer(name, dtype):
+    """Output position o samples around o*stride - pad + tap*dilation whichever size formula is in
+    force, and the dilation-aware size never exceeds the dilation-blind one: the layer with
+    `standard_output_size` is the reference's layer cropped to the leading positions of every axis.
+    So the oracle, run at the reference's size with grad_output zero outside the crop, fixes the
+    output, grad_input and grad_weight, and (cropped) grad_offset."""
+    dcn = _dcn()
+    c = make_case(*SMALL_CASES[name], dtype=dtype, seed=11)
+    nd = c["nd"]
+    std = dcn.output_size(c["ins"], c["k"], c["stride"], c["pad"], c["dil"], standard=True)
+    assert all(1 <= s <= o for s, o in zip(std, c["outs"]))
+    crop = (slice(None), slice(None)) + tuple(slice(0, s) for s in std)
+    gout_full = torch.zeros_like(c["gout"])
+    gout_full[crop] = c["gout"][crop]
+    co = dict(c, gout=gout_full)
+    want_out, want_gin, want_goff, want_gw, want_gb = run_oracle(co)
+
+    fn = dcn.ConvOffset3dFunction if nd == 3 else dcn.ConvOffset2dFunction
+    dev = torch.device("cuda:0")
+    x, w, b = (c[k].to(dev).requires_grad_(True) for k in ("x", "w", "b"))
+    off = c["off"][crop].contiguous().to(dev).requires_grad_(True)
+    out = fn.apply(x, off, w, b, c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"], True)
+    assert tuple(out.shape[2:]) == std
+    out.backward(c["gout"][crop].contiguous().to(dev))
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert rel_err(out, want_out[crop]) <= tol["fwd"]
+    assert rel_err(x.grad, want_gin) <= tol["grad"]
+    assert rel_err(off.grad, want_goff[crop]) <= tol["grad"]
+    assert rel_err(w.grad, want_gw) <= tol["grad"]
+    assert rel_err(b.grad, want_gb) <= tol["grad"]
+
+
+@pytest.mark.parametrize("nd", [2, 3])
+def test_standard_output_size_zero_offsets_equal_dilated_convolution(nd):
+    """With zero offsets and the dilation-aware size the layer is torch's dilated convolution."""
+    dcn = _dcn()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(5)
+    ins = (9, 10) if nd == 2 else (7, 8, 9)
+    Layer = dcn.ConvOffset2dPack if nd == 2 else dcn.ConvOffset3dPack
+    layer = Layer(6, 8, 3, stride=1, padding=2, dilation=2, channel_per_group=3, groups=2, zero_init_offset=True,
+                  device=dev, dtype=torch.float64, standard_output_size=True)
+    x = torch.randn((2, 6) + ins, device=dev, dtype=torch.float64, requires_grad=True)
+    out = layer(x)
+    conv = torch.nn.functional.conv2d if nd == 2 else torch.nn.functional.conv3d
+    x2 = x.detach().clone().requires_grad_(True)
+    w2 = layer.weight.detach().clone().requires_grad_(True)
+    want = conv(x2, w2, layer.bias.detach(), stride=1, padding=2, dilation=2, groups=2)
+    assert out.shape == want.shape
+    g = torch.randn_like(want)
+    out.backward(g)
+    want.backward(g)
+    assert rel_err(out, want.detach().cpu()) <= 1e-10
+    assert rel_err(x.grad, x2.grad.cpu()) <= 1e-10
+    assert rel_err(layer.weight.grad, w2.grad.cpu()) <= 1e-10
+
+
 class _OracleLayer(torch.autograd.Function):
     """The CPU oracle as an autograd node, so that a CPU graph (offset convolution -> layer) can be
     differentiated end to end as the reference for the Pack modules."""

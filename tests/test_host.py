@@ -143,3 +143,26 @@ def test_pack_modules_construction():
         dcn.ConvOffset2dPack(6, 4, 3, channel_per_group=4)
     with pytest.raises(RuntimeError):          # no CPU path: the layer itself needs the GPU
         m2(torch.randn(1, 4, 5, 5))
+
+
+def test_standard_output_size_formula():
+    from deform_conv3d_pytorch_op_amd import output_size
+    # reference formula: dilation ignored
+    assert output_size((8, 8, 8), (3, 3, 3), (1, 1, 1), (3, 3, 3)) == (12, 12, 12)
+    # dilation-aware: torch's convolution size
+    assert output_size((8, 8, 8), (3, 3, 3), (1, 1, 1), (3, 3, 3), (3, 3, 3), standard=True) == (8, 8, 8)
+    for i, k, s, p, d in [(10, 3, 2, 1, 2), (7, 1, 3, 0, 4), (9, 2, 1, 0, 3), (16, 5, 2, 4, 2)]:
+        want = torch.nn.functional.conv1d(torch.zeros(1, 1, i), torch.zeros(1, 1, k), stride=s, padding=p, dilation=d).shape[-1]
+        assert output_size((i,), (k,), (s,), (p,), (d,), standard=True) == (want,)
+        # never larger than the reference's size, equal for dilation 1
+        assert want <= output_size((i,), (k,), (s,), (p,))[0]
+        assert output_size((i,), (k,), (s,), (p,), (1,), standard=True) == output_size((i,), (k,), (s,), (p,))
+
+
+def test_pack_module_offset_convolution_follows_output_size_mode():
+    from deform_conv3d_pytorch_op_amd import ConvOffset2dPack
+    blind = ConvOffset2dPack(4, 4, 3, padding=2, dilation=2)
+    std = ConvOffset2dPack(4, 4, 3, padding=2, dilation=2, standard_output_size=True)
+    assert blind.conv_offset.dilation == (1, 1) and std.conv_offset.dilation == (2, 2)
+    x = torch.zeros(1, 4, 9, 9)
+    assert blind.conv_offset(x).shape[2:] == (11, 11) and std.conv_offset(x).shape[2:] == (9, 9)
