@@ -50,10 +50,22 @@ template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp)
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 constexpr int TAP_PAD = 8;      // zero tap slabs behind the last group: an MFMA pass may start up to 7 taps before the end
+// Elements of the per-chunk weight slabs of the fused backward kernel (pack_weight_kernel, 4-channel
+// chunks) for `slabs` slabs.
+template <typename T> size_t packed_weight_elems(int M, int kV, size_t slabs) {
+    const int KL = Mma<T>::KL, TP = Mma<T>::TN / 4;
+    return slabs * ((kV + TP - 1) / TP) * (size_t)(((M + KL - 1) / KL + 7) / 8 * 8) * 64;
+}
+// Either weight layout of backward_input_offset fits.  The slab count of the packed one depends on
+// the deformable groups, which the workspace query is not told: it is bounded by their largest
+// possible number, C_in.
 template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G) {
     int Mp, Cgp;
     bwd_data_weight_pad<T>(M, Cg, Mp, Cgp);
-    return align256(((size_t)G * kV + TAP_PAD) * Mp * Cgp * sizeof(T));
+    const size_t plain = ((size_t)G * kV + TAP_PAD) * Mp * Cgp;
+    const size_t C_in = (size_t)Cg * G;
+    const size_t packed = packed_weight_elems<T>(M, kV, C_in / 4 + C_in + G + 1);
+    return align256((plain > packed ? plain : packed) * sizeof(T));
 }
 template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G) {
     const int M = C_out / G, Cg = C_in / G;
@@ -341,12 +353,6 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     T* wt = static_cast<T*>(ws);
     T* in_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes);
     T* gin_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes + tbytes);
-    if (int rc = relayout<T>(P, w, wt, 1, s)) return rc;
-    {   // zero tap slabs behind the last group
-        const size_t used = (size_t)P.G * P.kV * P.Mp * P.Cgp, pad = (size_t)TAP_PAD * P.Mp * P.Cgp;
-        hipLaunchKernelGGL(fill_zero_kernel<T>, dim3((unsigned)((pad + 255) / 256)), dim3(256), 0, s, wt + used, pad);
-        if (int rc = check_launch("fill_zero_kernel")) return rc;
-    }
     const int TN = Mma<T>::TN;
     const int mk = bwd_data_mk<T>(P.M);
     float* wmax = reinterpret_cast<float*>(gin_cl);     // the channels-last gradient buffer is free on the LDS paths
@@ -368,6 +374,12 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         Ph.cchunk = 4;
         if (fixed) Ph.hstride = FUSED_HS;
         const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + tables;
+        {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
+            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in);
+            const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
+            hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt);
+            if (int rc = check_launch("pack_weight_kernel")) return rc;
+        }
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
         // wastes least of the last round (one workgroup per CU at this LDS size)
@@ -392,7 +404,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         // grad_output operand held in registers when its reduction steps fit (M <= 64 float, 128 double)
         const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32;
 #define DCN_LAUNCH_FUSED(BREG_, HS_, NW_)                                                                              \
-    launch_halo(backward_input_halo_kernel<T, ND, 4, true, BREG_, HS_, NW_>, "backward_input_halo_kernel", hgrid, NW_ * 64, \
+    launch_halo(backward_input_halo_kernel<T, ND, 4, true, BREG_, HS_, NW_, true>, "backward_input_halo_kernel", hgrid, NW_ * 64, \
                 lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit)
         if (nw == 8) {
             if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 8);
@@ -406,6 +418,12 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     }
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
+    if (int rc = relayout<T>(P, w, wt, 1, s)) return rc;
+    {   // zero tap slabs behind the last group
+        const size_t used = (size_t)P.G * P.kV * P.Mp * P.Cgp, pad = (size_t)TAP_PAD * P.Mp * P.Cgp;
+        hipLaunchKernelGGL(fill_zero_kernel<T>, dim3((unsigned)((pad + 255) / 256)), dim3(256), 0, s, wt + used, pad);
+        if (int rc = check_launch("fill_zero_kernel")) return rc;
+    }
     hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
     Params Ph = P;

@@ -34,6 +34,41 @@ __global__ void relayout_weight_kernel(Params P, const T* __restrict__ W, T* __r
     }
 }
 
+// Backward-data weights of the halo kernels that take CCH-channel chunks of a segment (the channels
+// shared by one deformable group and one convolution group): one slab per chunk, in the order the
+// lanes of a wavefront consume it, Wp[slab][pass][k][lane].  Lane (q, j) of reduction step k in MFMA
+// pass `pass` holds W[m = k*KL + q][channel = first + j % CCH][tap = pass*TP + j / CCH], zero past
+// M, past the last tap and past the segment, so every operand load of the kernel is one contiguous
+// 64-element read (in [tap][m][channel] order the same load touches 16 separate cache lines).
+// A chunk that starts at channel c0 owns slab chunk_slot(c0): increasing in c0, by at least one per
+// chunk (c0 / CCH steps within a segment, one of the other terms at every segment start), so no two
+// chunks share a slab; some slabs stay unused.
+template <int CCH>
+__host__ __device__ inline int chunk_slot(int cpg, int Cg, int c0) { return c0 / CCH + c0 / cpg + c0 / Cg; }
+
+template <typename T, int CCH>
+__global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, TP = TN / CCH;
+    const int npass = (P.kV + TP - 1) / TP;
+    const int kst = ((P.M + KL - 1) / KL + 7) / 8 * 8;          // operand batches are 8 reduction steps
+    const size_t per_chunk = (size_t)npass * kst * 64;
+    const size_t total = (size_t)P.C_in * per_chunk;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int c0 = (int)(i / per_chunk);                    // candidate first channel of a chunk
+        const int seg_b = max(c0 / P.cpg * P.cpg, c0 / P.Cg * P.Cg);
+        if ((c0 - seg_b) % CCH) continue;
+        const int seg_e = min((c0 / P.cpg + 1) * P.cpg, (c0 / P.Cg + 1) * P.Cg);
+        const size_t r = i % per_chunk;
+        const int lane = (int)(r % 64), k = (int)((r / 64) % kst), pass = (int)(r / 64 / kst);
+        const int q = lane / TN, j = lane % TN;
+        const int m = k * KL + q, tap = pass * TP + j / CCH, c = c0 + j % CCH, g = c0 / P.Cg;
+        T v = 0;
+        if (m < P.M && tap < P.kV && c < seg_e) v = W[(((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap];
+        Wp[(size_t)chunk_slot<CCH>(P.cpg, P.Cg, c0) * per_chunk + r] = v;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Forward: out[n][g*M + m][pos] = sum_{cl,tap} W[g*M+m][cl][tap] * sample(in[n][g*Cg+cl], tap, pos)  (+ bias)
 // replaces deformable_im2col + the per-group Sgemm (deform3d/lib/deform_conv3d_cuda.cpp:110-148,
@@ -745,7 +780,9 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // NW wavefronts per workgroup (8; 4 where only a smaller block of positions has a halo that fits).
 // HS > 0 fixes the plane stride at compile time (the host then plans with hstride = HS): the plane
 // of a channel becomes an immediate offset of the LDS instructions instead of address arithmetic.
-template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW>
+// PACKW: the weights come in the per-chunk lane order of pack_weight_kernel instead of
+// [g][tap][m][channel].
+template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false>
 __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
@@ -801,7 +838,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     int chunk_no = 0;
     // this lane's row of the A operand: (tap slot, channel) = (j / CCH, j % CCH)
     const int a_tl = j / CCH, a_c = j % CCH;
-    const unsigned a_off = ((unsigned)a_tl * P.Mp + q) * P.Cgp + a_c;      // lane offset inside a tap group's weight slabs
+    const unsigned a_off = PACKW ? (unsigned)lane : ((unsigned)a_tl * P.Mp + q) * P.Cgp + a_c;      // lane offset inside a tap group's weight slabs
 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
@@ -863,10 +900,11 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             // the matrix pipe works behind the vector work of the scatter instead of before it.
             // Operands arrive in batches of AB reduction steps, loaded one tap slot ahead of use.
             constexpr int MPR = AB / RPS;                              // MFMAs per accumulator register walked
-            const size_t wstep = (size_t)KL * P.Cgp;
-            const size_t wpass = (size_t)TP * P.Mp * P.Cgp;            // weight slabs of one pass
             const int ksteps = (P.M + KL - 1) / KL;
-            const T* wchunk = Wt + ((size_t)g * P.kV * P.Mp) * P.Cgp + (cc0 - g * P.Cg);      // uniform; lanes add a_off
+            const size_t wstep = PACKW ? (size_t)64 : (size_t)KL * P.Cgp;
+            const size_t wpass = PACKW ? (size_t)((ksteps + 7) / 8 * 8) * 64 : (size_t)TP * P.Mp * P.Cgp;   // weights of one pass
+            const T* wchunk = PACKW ? Wt + (size_t)chunk_slot<CCH>(P.cpg, P.Cg, cc0) * ((P.kV + TP - 1) / TP) * wpass
+                                    : Wt + ((size_t)g * P.kV * P.Mp) * P.Cgp + (cc0 - g * P.Cg);      // uniform; lanes add a_off
             // (k0 passes through an empty asm: what is derived from it is then computed where it is
             // used instead of being hoisted out of the loops into hundreds of long-lived registers)
             auto load_batch = [&](T* a_nx, T* b_nx, const T* wp, int k0) {      // rows past M are zero padding
