@@ -50,10 +50,10 @@ template <typename T> void bwd_data_weight_pad(int M, int Cg, int& Mp, int& Cgp)
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 constexpr int TAP_PAD = 8;      // zero tap slabs behind the last group: an MFMA pass may start up to 7 taps before the end
-// Elements of the per-chunk weight slabs of the fused backward kernel (pack_weight_kernel, 4-channel
-// chunks) for `slabs` slabs.
-template <typename T> size_t packed_weight_elems(int M, int kV, size_t slabs) {
-    const int KL = Mma<T>::KL, TP = Mma<T>::TN / 4;
+// Elements of the per-chunk weight slabs of the fused backward kernel (pack_weight_kernel, chunks of
+// `cch` channels) for `slabs` slabs.
+template <typename T> size_t packed_weight_elems(int M, int kV, size_t slabs, int cch) {
+    const int KL = Mma<T>::KL, TP = Mma<T>::TN / cch;
     return slabs * ((kV + TP - 1) / TP) * (size_t)(((M + KL - 1) / KL + 7) / 8 * 8) * 64;
 }
 // Either weight layout of backward_input_offset fits.  The slab count of the packed one depends on
@@ -64,7 +64,9 @@ template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G)
     bwd_data_weight_pad<T>(M, Cg, Mp, Cgp);
     const size_t plain = ((size_t)G * kV + TAP_PAD) * Mp * Cgp;
     const size_t C_in = (size_t)Cg * G;
-    const size_t packed = packed_weight_elems<T>(M, kV, C_in / 4 + C_in + G + 1);
+    const size_t packed4 = packed_weight_elems<T>(M, kV, C_in / 4 + C_in + G + 1, 4);
+    const size_t packed8 = packed_weight_elems<T>(M, kV, C_in / 8 + C_in + G + 1, 8);
+    const size_t packed = packed4 > packed8 ? packed4 : packed8;
     return align256((plain > packed ? plain : packed) * sizeof(T));
 }
 template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G) {
@@ -155,6 +157,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
 //   DCN_FUSED_WAVES=4      fused backward kernel with four wavefronts per workgroup even where eight fit
+//   DCN_FUSED_CHUNK=4      fused backward kernel with 4-channel chunks also where it would take 8 (2-D layers)
 static size_t env_kb(const char* name, int dflt) {
     const char* e = getenv(name);
     const int v = e ? atoi(e) : dflt;
@@ -183,6 +186,10 @@ static int wide_forward() {      // 0 never, 1 when it pays, 2 whenever the halo
         return !e ? 1 : atoi(e) == 512 ? 0 : atoi(e) == 1024 ? 2 : 1;
     }();
     return v;
+}
+static bool fused_chunk8() {      // DCN_FUSED_CHUNK=4: never take 8-channel chunks in the fused backward kernel
+    static const int v = [] { const char* e = getenv("DCN_FUSED_CHUNK"); return (e && atoi(e) == 4) ? 0 : 1; }();
+    return v != 0;
 }
 static int fused_first_waves() {
     static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : 8; }();
@@ -371,19 +378,28 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const bool fixed = Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
         if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
         if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) < 4) continue;
-        Ph.cchunk = 4;
-        if (fixed) Ph.hstride = FUSED_HS;
-        const size_t lds = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + tables;
+        // Channels per chunk: 8 where that takes fewer MFMA passes per channel (a pass holds TN / CCH
+        // taps: the 9 taps of a 3x3 kernel are 2 float passes per 4 channels or 3 per 8) and the
+        // planes of 8 channels fit, which the small halos of 2-D layers allow.
+        const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;
+        auto passes = [&](int c) { const int tp = Mma<T>::TN / c; return (P.kV + tp - 1) / tp; };
+        const bool eight = ND == 2 && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
+                           (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 8;
+        const int cch = eight ? 8 : 4;
+        Ph.cchunk = cch;
+        if (fixed && !eight) Ph.hstride = FUSED_HS;
+        const size_t lds = (size_t)cch * Ph.hstride * (8 + sizeof(T)) + tables;
         {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
-            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in);
+            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in, cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
-            hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt);
+            if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), dim3(blocks), dim3(256), 0, s, P, w, wt);
+            else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt);
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
         // wastes least of the last round (one workgroup per CU at this LDS size)
-        const int nchunks = ((P.cpg < P.Cg ? P.cpg : P.Cg) + 3) / 4;
+        const int nchunks = (seg + cch - 1) / cch;
         const long long items = (long long)Ph.N * Ph.tiles * Ph.DG;
         const int cus = cu_count();
         int csplit = 1;
@@ -401,11 +417,17 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (int rc = check_launch("fill_zero_kernel")) return rc;
         }
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG * csplit);
-        // grad_output operand held in registers when its reduction steps fit (M <= 64 float, 128 double)
-        const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= 32;
-#define DCN_LAUNCH_FUSED(BREG_, HS_, NW_)                                                                              \
-    launch_halo(backward_input_halo_kernel<T, ND, 4, true, BREG_, HS_, NW_, true>, "backward_input_halo_kernel", hgrid, NW_ * 64, \
+        // grad_output operand held in registers when its reduction steps fit: 8 per tap slot of a pass
+        // (M <= 64 float, 128 double with 4-channel chunks)
+        const int slot_regs = (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
+        const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= Mma<T>::NACC / slot_regs * 8;
+#define DCN_LAUNCH_FUSED_C(CCH_, BREG_, HS_, NW_)                                                                     \
+    launch_halo(backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true>, "backward_input_halo_kernel", hgrid, NW_ * 64, \
                 lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit)
+#define DCN_LAUNCH_FUSED(BREG_, HS_, NW_) DCN_LAUNCH_FUSED_C(4, BREG_, HS_, NW_)
+        if constexpr (ND == 2) {
+            if (eight) return breg ? DCN_LAUNCH_FUSED_C(8, true, 0, 8) : DCN_LAUNCH_FUSED_C(8, false, 0, 8);
+        }
         if (nw == 8) {
             if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 8);
             if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 8);
@@ -415,6 +437,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 4);
         return DCN_LAUNCH_FUSED(false, 0, 4);
 #undef DCN_LAUNCH_FUSED
+#undef DCN_LAUNCH_FUSED_C
     }
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter

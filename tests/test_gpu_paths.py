@@ -10,6 +10,7 @@ settings, each in a process of its own (the knobs are read once per process):
   DCN_COORD=separate   grad_offset from the channels-last kernel, grad_input from the scatter-only kernel
   DCN_CSPLIT=1 / 4     channel chunks of the fused backward kernel on one / four workgroups
   DCN_FUSED_WAVES=4    the fused backward kernel's four-wavefront shape (otherwise only strided full-size cases use it)
+  DCN_FUSED_CHUNK=4    the fused backward kernel with 4-channel chunks also for 2-D layers (which otherwise take 8)
 """
 import os
 import subprocess
@@ -29,6 +30,7 @@ SETTINGS = [
     {"DCN_FORWARD_WG": "512", "DCN_CSPLIT": "1"},
     {"DCN_COORD": "separate"},
     {"DCN_FUSED_WAVES": "4"},
+    {"DCN_FUSED_CHUNK": "4"},
 ]
 
 
