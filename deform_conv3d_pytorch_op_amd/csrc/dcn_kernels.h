@@ -858,6 +858,13 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             const T b = gb[ok ? b_off : pos];
             return (!masked || (ok && valid)) ? b : (T)0;
         };
+        // The same operand for the batches of the GEMM loops: the row base advances in scalar
+        // registers, clamped at the last real step (further steps of a batch meet zero weight rows
+        // and re-read that step), and the lane adds a 32-bit byte offset, so that a load costs a
+        // few scalar instructions and one select instead of 64-bit address arithmetic per lane.
+        const int klast = (P.M + KL - 1) / KL - 1;
+        const unsigned b_byte = b_off * (unsigned)sizeof(T);
+        const unsigned b_byte_last = (klast * KL + q < P.M ? b_off : pos) * (unsigned)sizeof(T);
         T b_reg[BREG ? NS * AB : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
         if constexpr (BREG) {
@@ -910,10 +917,14 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             auto load_batch = [&](T* a_nx, T* b_nx, const T* wp, int k0) {      // rows past M are zero padding
                 asm volatile("" : "+s"(k0));
                 const T* wb = wp + (size_t)k0 * wstep;                 // one 64-bit product per batch; the row offsets below are loop invariants
+                const char* gk = reinterpret_cast<const char*>(gbase + (size_t)min(k0, klast) * gstep);
 #pragma unroll
                 for (int k = 0; k < AB; ++k) {
                     a_nx[k] = (wb + (unsigned)k * (unsigned)wstep)[a_off];
-                    if constexpr (!BREG) b_nx[k] = load_b(k0 + k, false);
+                    if constexpr (!BREG) {
+                        b_nx[k] = *reinterpret_cast<const T*>(gk + (k0 + k >= klast ? b_byte_last : b_byte));
+                        gk += k0 + k < klast ? gstep * sizeof(T) : (size_t)0;
+                    }
                 }
             };
             // steps [k_begin, ksteps) of one pass in a software-pipelined loop of their own: the whole
