@@ -868,10 +868,21 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         T b_reg[BREG ? NS * AB : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
         if constexpr (BREG) {
+            // held unmasked (rows past M meet zero weight rows, columns outside the volume are never
+            // used): a masked load becomes a conditional one, issued alone with a full wait behind it
+            // (the last step passes through an empty asm: the per-step selects derived from it are
+            // then computed here, not hoisted out of the group loop into registers that stay live
+            // through the whole kernel)
+            int kl = klast;
+            asm volatile("" : "+s"(kl));
+            const char* gk = reinterpret_cast<const char*>(gbase);
 #pragma unroll
-            for (int k = 0; k < NS * AB; ++k) b_reg[k] = load_b(k, true);
+            for (int k = 0; k < NS * AB; ++k) {
+                b_reg[k] = *reinterpret_cast<const T*>(gk + (k >= kl ? b_byte_last : b_byte));
+                gk += k < kl ? gstep * sizeof(T) : (size_t)0;
+            }
 #pragma unroll
-            for (int k = 0; k < NS * AB; ++k) sabs += fabsf((float)b_reg[k]);
+            for (int k = 0; k < NS * AB; ++k) sabs += (valid && (k < kl || (k == kl && kl * KL + q < P.M))) ? fabsf((float)b_reg[k]) : 0.f;
         } else {
             for (int k = 0; k * KL < P.M; ++k) sabs += fabsf((float)load_b(k, true));
         }
