@@ -571,6 +571,9 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     if (int rc = validate(g, P)) return rc;
     if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     if ((long long)P.outV * P.C_out > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one output sample exceeds 2^31 elements");
+    // the kernel addresses both operands by 32-bit byte offsets from the sample's base
+    if ((unsigned long long)P.inV * P.C_in * sizeof(T) >= (1ull << 32) || (unsigned long long)P.outV * P.C_out * sizeof(T) >= (1ull << 32))
+        return fail(DCN_E_ARGUMENT, "one sample of the input or of grad_output reaches 4 GiB");
     int MT;
     bww_plan<T>(P, MT, P.mchunks, P.nctiles, P.nsplit);
     const long long resident = MT == 1 ? bww_resident<T, ND, 1>() : MT == 2 ? bww_resident<T, ND, 2>() : bww_resident<T, ND, 4>();

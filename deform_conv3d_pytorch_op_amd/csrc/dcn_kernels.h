@@ -1094,14 +1094,20 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                             for (int rr = 0; rr < RPS; ++rr)
                                 gvc[rr] = (MM::row(ts * RPS + rr, q) % CCH) < nch ? d[ts * RPS + rr] : (T)0;
+                            // every corner's read is issued before the first is used: one wait for
+                            // the LDS queue (the previous slot's adds are ahead in it) instead of one
+                            // per pair of reads
+                            T vv[NC][RPS];
+#pragma unroll
+                            for (int i = 0; i < NC; ++i)
+#pragma unroll
+                                for (int rr = 0; rr < RPS; ++rr) vv[i][rr] = in_cell[i][MM::row(ts * RPS + rr, q) % CCH];
+                            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                             for (int i = 0; i < NC; ++i) {
-                                T vv[RPS];
-#pragma unroll
-                                for (int rr = 0; rr < RPS; ++rr) vv[rr] = in_cell[i][MM::row(ts * RPS + rr, q) % CCH];
                                 T acc_ = 0;
 #pragma unroll
-                                for (int rr = 0; rr < RPS; ++rr) acc_ += gvc[rr] * vv[rr];
+                                for (int rr = 0; rr < RPS; ++rr) acc_ += gvc[rr] * vv[i][rr];
                                 gsum[i] = acc_;
                             }
                         }
@@ -1208,11 +1214,15 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
                                                              const T* __restrict__ gout_cl, T* __restrict__ partial) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
-    __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // corner voxel index * C_in, 0 when the sample is dead
-    __shared__ __align__(16) T sF[WAVES][TN][4];             // f[ND]; [3] = 1 when the sample is live
+    // geometry record of a (tap, position), written once per slab and read by every reduction step
+    __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // byte offset of each corner's channel 0 inside the sample, 0 when the sample is dead
+    __shared__ __align__(16) T sCw[WAVES][TN][NC];           // interpolation weight of each corner, 0 when the sample is dead
+    __shared__ unsigned sLive[WAVES][TN];                    // 1 when the sample is live
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sAcc = reinterpret_cast<T*>(smem_raw);                // [WAVES][TN][TN + 1]: the wavefronts' partial tiles, one row tile at a time
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // (the wavefront number as a scalar: the slab, the sample and the operand bases derived from it
+    // then live in scalar registers and the loads take the scalar-base + 32-bit-offset form)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane % TN, q = lane / TN;
 
     // 1-D grid of nctiles * mchunks * nsplit * kV workgroups in an XCD-contiguous order with the tap
@@ -1251,13 +1261,17 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
     const int m_base = mchunk * MT * TN;
     const bool chan_ok = c0 + j < ce;
     const unsigned cj = (unsigned)min(c0 + j, P.C_in - 1);          // clamped: dead lanes still load legally
-    unsigned mrow[MT];
+    // operands are addressed by 32-bit byte offsets from the sample's base (the host checks that a
+    // sample of either tensor stays below 4 GiB)
+    const unsigned cjB = cj * (unsigned)sizeof(T);
+    const unsigned cinB = (unsigned)P.C_in * (unsigned)sizeof(T), rowB = (unsigned)P.C_out * (unsigned)sizeof(T);
+    unsigned mrowB[MT];
     bool m_ok[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = m_base + mt * TN + j;
         m_ok[mt] = m < P.M;
-        mrow[mt] = (unsigned)(g * P.M + min(m, P.M - 1));
+        mrowB[mt] = (unsigned)(g * P.M + min(m, P.M - 1)) * (unsigned)sizeof(T);
     }
 
     const int slabs_per_sample = (P.outV + TN - 1) / TN;
@@ -1280,24 +1294,35 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (q == 0) {
+            T cw[NC];                              // multiplied in the reference's order (w_l * w_h * w_w)
+            if constexpr (ND == 3) {
+                const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+            } else {
+                const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+            }
 #pragma unroll
-            for (int i = 0; i < NC; ++i) sIdx[wave][j][i] = live ? t.idx[i] * (unsigned)P.C_in : 0u;
+            for (int i = 0; i < NC; ++i) sIdx[wave][j][i] = live ? t.idx[i] * cinB : 0u;
 #pragma unroll
-            for (int a = 0; a < ND; ++a) sF[wave][j][a] = t.f[a];
-            sF[wave][j][3] = live ? (T)1 : (T)0;
+            for (int i = 0; i < NC; ++i) sCw[wave][j][i] = live ? cw[i] : (T)0;
+            sLive[wave][j] = live ? 1u : 0u;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        const T* in_n = in_cl + (size_t)n * P.inV * P.C_in + cj;
-        const T* go_n = gout_cl + (size_t)n * P.outV * P.C_out;
+        const char* in_n = reinterpret_cast<const char*>(in_cl + (size_t)n * P.inV * P.C_in);        // scalar bases
+        const char* go_n = reinterpret_cast<const char*>(gout_cl + (size_t)n * P.outV * P.C_out);
+        const unsigned a_first = (p0 + (unsigned)q) * rowB;          // grad_output row of this lane's position in step 0
+        const unsigned a_last = (P.outV - 1) * rowB;                 // positions past the end re-read the last row (masked below)
         // reduction over the slab's positions, software pipelined: while step ks is interpolated and
         // multiplied, the geometry record, the corner values and the grad_output rows of step ks + 1
         // are already in flight
         constexpr int NK = TN / KL;
         constexpr int DEPTH = 1;                    // steps in flight ahead of the one being multiplied (2 costs a wavefront of occupancy and is slower)
-        T cn[DEPTH][NC], an[DEPTH][MT], fn[DEPTH][ND];
+        T cn[DEPTH][NC], an[DEPTH][MT], wn[DEPTH][NC];
         bool lvn[DEPTH], okn[DEPTH];
         auto fetch = [&](int ks, int slot_) {
             const int pp = ks * KL + q;             // position of the slab this lane group works on
@@ -1305,31 +1330,35 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 #pragma unroll
             for (int i = 0; i < NC; ++i) ix[i] = sIdx[wave][pp][i];
 #pragma unroll
-            for (int a_ = 0; a_ < ND; ++a_) fn[slot_][a_] = sF[wave][pp][a_];
-            lvn[slot_] = sF[wave][pp][3] != (T)0;
-            const unsigned pg = min(p0 + (unsigned)pp, P.outV - 1);
+            for (int i = 0; i < NC; ++i) wn[slot_][i] = sCw[wave][pp][i];
+            lvn[slot_] = sLive[wave][pp] != 0u;
             okn[slot_] = p0 + (unsigned)pp < P.outV;
-            const T* grow = go_n + (size_t)pg * P.C_out;
+            const unsigned ao = min(a_first + (unsigned)(ks * KL) * rowB, a_last);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) an[slot_][mt] = grow[mrow[mt]];   // A[row = m][k = position]; legal for every lane
-            load_corners<T, ND>(in_n, ix, cn[slot_]);                         // dead samples read voxel 0
+            for (int mt = 0; mt < MT; ++mt)         // A[row = m][k = position]; legal for every lane
+                an[slot_][mt] = *reinterpret_cast<const T*>(go_n + (ao + mrowB[mt]));
+#pragma unroll
+            for (int i = 0; i < NC; ++i)            // dead samples read voxel 0
+                cn[slot_][i] = *reinterpret_cast<const T*>(in_n + (ix[i] + cjB));
         };
 #pragma unroll
         for (int d0 = 0; d0 < DEPTH; ++d0) fetch(d0, d0);
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks) {
             const int sl = ks % DEPTH;
-            T cc[NC], ac[MT], fc[ND];
+            T cc[NC], ac[MT], wc[NC];
 #pragma unroll
             for (int i = 0; i < NC; ++i) cc[i] = cn[sl][i];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) ac[mt] = an[sl][mt];
 #pragma unroll
-            for (int a_ = 0; a_ < ND; ++a_) fc[a_] = fn[sl][a_];
+            for (int i = 0; i < NC; ++i) wc[i] = wn[sl][i];
             const bool lvc = lvn[sl], okc = okn[sl];
             if (ks + DEPTH < NK) fetch(ks + DEPTH, sl);
             __builtin_amdgcn_sched_barrier(0);      // later steps' loads are issued before this step's arithmetic
-            const T v = interp<T, ND>(cc, fc);
+            T v = wc[0] * cc[0];                    // weighted corner sum, as the reference's sampler forms it
+#pragma unroll
+            for (int i = 1; i < NC; ++i) v += wc[i] * cc[i];
             const T b = (lvc && chan_ok) ? v : (T)0;                                   // B[k = position][col = channel j]
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma((okc && m_ok[mt]) ? ac[mt] : (T)0, b, acc[mt]);
