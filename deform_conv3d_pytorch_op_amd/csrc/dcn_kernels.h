@@ -1259,18 +1259,15 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
     for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
 
     const int m_base = mchunk * MT * TN;
-    const bool chan_ok = c0 + j < ce;
     const unsigned cj = (unsigned)min(c0 + j, P.C_in - 1);          // clamped: dead lanes still load legally
     // operands are addressed by 32-bit byte offsets from the sample's base (the host checks that a
     // sample of either tensor stays below 4 GiB)
     const unsigned cjB = cj * (unsigned)sizeof(T);
     const unsigned cinB = (unsigned)P.C_in * (unsigned)sizeof(T), rowB = (unsigned)P.C_out * (unsigned)sizeof(T);
     unsigned mrowB[MT];
-    bool m_ok[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = m_base + mt * TN + j;
-        m_ok[mt] = m < P.M;
         mrowB[mt] = (unsigned)(g * P.M + min(m, P.M - 1)) * (unsigned)sizeof(T);
     }
 
@@ -1321,9 +1318,9 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
         // multiplied, the geometry record, the corner values and the grad_output rows of step ks + 1
         // are already in flight
         constexpr int NK = TN / KL;
-        constexpr int DEPTH = 1;                    // steps in flight ahead of the one being multiplied (2 costs a wavefront of occupancy and is slower)
+        constexpr int DEPTH = 1;                    // steps in flight ahead of the one being multiplied (2 is no faster)
         T cn[DEPTH][NC], an[DEPTH][MT], wn[DEPTH][NC];
-        bool lvn[DEPTH], okn[DEPTH];
+        bool lvn[DEPTH];
         auto fetch = [&](int ks, int slot_) {
             const int pp = ks * KL + q;             // position of the slab this lane group works on
             unsigned ix[NC];
@@ -1332,7 +1329,6 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 #pragma unroll
             for (int i = 0; i < NC; ++i) wn[slot_][i] = sCw[wave][pp][i];
             lvn[slot_] = sLive[wave][pp] != 0u;
-            okn[slot_] = p0 + (unsigned)pp < P.outV;
             const unsigned ao = min(a_first + (unsigned)(ks * KL) * rowB, a_last);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)         // A[row = m][k = position]; legal for every lane
@@ -1353,15 +1349,18 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
             for (int mt = 0; mt < MT; ++mt) ac[mt] = an[sl][mt];
 #pragma unroll
             for (int i = 0; i < NC; ++i) wc[i] = wn[sl][i];
-            const bool lvc = lvn[sl], okc = okn[sl];
+            const bool lvc = lvn[sl];
             if (ks + DEPTH < NK) fetch(ks + DEPTH, sl);
             __builtin_amdgcn_sched_barrier(0);      // later steps' loads are issued before this step's arithmetic
             T v = wc[0] * cc[0];                    // weighted corner sum, as the reference's sampler forms it
 #pragma unroll
             for (int i = 1; i < NC; ++i) v += wc[i] * cc[i];
-            const T b = (lvc && chan_ok) ? v : (T)0;                                   // B[k = position][col = channel j]
+            // B[k = position][col = channel j], exactly zero for a dead sample and for a position past
+            // the end.  Nothing else is masked: a row of A only reaches its own row of the tile and a
+            // column of B its own column, and rows past M / columns past the segment are not stored.
+            const T b = lvc ? v : (T)0;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma((okc && m_ok[mt]) ? ac[mt] : (T)0, b, acc[mt]);
+            for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(ac[mt], b, acc[mt]);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
