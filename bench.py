@@ -34,8 +34,8 @@ PEAK_HBM_GBS = 8000.0
 # that were profiled; otherwise `traffic` is null.
 MEASURED_TRAFFIC_BYTES = {
     ("c4", "forward"): 0.524e9,
-    ("c4", "backward_input_offset"): 1.981e9,
-    ("c4", "backward_weight"): 1.195e9,
+    ("c4", "backward_input_offset"): 1.992e9,
+    ("c4", "backward_weight"): 1.051e9,
 }
 
 # name: (nd, N, C_in, C_out, in, k, stride, pad, dil, cpg, groups, offset scale / dist, dtype)
