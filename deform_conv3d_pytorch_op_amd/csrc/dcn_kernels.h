@@ -917,7 +917,22 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
             for (int k = 0; k < NS * AB; ++k) sabs += (valid && (k < kl || (k == kl && kl * KL + q < P.M))) ? fabsf((float)b_reg[k]) : 0.f;
         } else {
-            for (int k = 0; k * KL < P.M; ++k) sabs += fabsf((float)load_b(k, true));
+            // unconditional loads, eight in flight, masked when they are summed (a masked load
+            // becomes a conditional one that is waited for on its own)
+            const char* gk = reinterpret_cast<const char*>(gbase);
+            for (int k0 = 0; k0 <= klast; k0 += AB) {
+                T bv[AB];
+#pragma unroll
+                for (int k = 0; k < AB; ++k) {
+                    bv[k] = *reinterpret_cast<const T*>(gk + (k0 + k >= klast ? b_byte_last : b_byte));
+                    gk += k0 + k < klast ? gstep * sizeof(T) : (size_t)0;
+                }
+#pragma unroll
+                for (int k = 0; k < AB; ++k) {
+                    const int kk_ = k0 + k;
+                    sabs += (valid && (kk_ < klast || (kk_ == klast && klast * KL + q < P.M))) ? fabsf((float)bv[k]) : 0.f;
+                }
+            }
         }
         // fixed-point exponent of this (workgroup, convolution group): terms are bounded by
         // 8 * max|W| * max_pos sum_m |grad_output|
