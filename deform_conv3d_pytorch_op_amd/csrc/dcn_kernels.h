@@ -251,9 +251,11 @@ __device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, 
             T val[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) val[k] = ch[g[k]];              // four loads in flight
+            // unconditional stores (past the last voxel: into the plane's last padding cell, which is
+            // never read), so that the loads above are not folded into conditional blocks and waited
+            // for one by one
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (v0 + WGS * k < P.hvol) sIn[c * P.hstride + v0 + WGS * k] = val[k];
+            for (int k = 0; k < 4; ++k) sIn[c * P.hstride + (v0 + WGS * k < P.hvol ? v0 + WGS * k : P.hstride - 1)] = val[k];
         }
     }
 }
@@ -419,10 +421,18 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
                         wr += (size_t)KL * P.Mp;                           // rows past the chunk stay inside the padded weight
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt) a_next[mt] = wr[mt * TN];
+                        // (few accumulators: the compiler otherwise moves these loads behind the
+                        // first MFMA of the step, where they are waited for at once; pinned at the end
+                        // of the step they stay here and have the whole step to arrive)
+                        if constexpr (MT <= 2) __builtin_amdgcn_sched_barrier(0);
                         const T v = sample<T, ND>(plane, lidx, t.f);
                         const T b = (near && s * KL + q < nch) ? v : (T)0;
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a_cur[mt], b, acc[mt]);
+                        if constexpr (MT <= 2) {
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(a_next[mt]));
+                        }
                         plane += KL * P.hstride;
                     }
                 }
