@@ -407,7 +407,26 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
                                 (size_t)mchunk * MT * TN + j;
                 // branch-free main loop: every lane reads LDS at a legal index and the value is
                 // masked afterwards; the weights of the next step are fetched one step ahead
-                {
+                if constexpr (MT <= 2 && NW == 16) {
+                    // few accumulators, four wavefronts per SIMD: the step's own weights are requested at
+                    // its top and a scheduling barrier keeps the loads there (the LDS reads, the
+                    // interpolation and the other wavefronts cover their latency); the compiler otherwise
+                    // moves one of them between the two MFMAs, where it is waited for at once
+                    const T* plane = sIn;
+                    const T* wr = wrow;
+                    for (int s = 0; s < nsteps; ++s) {
+                        T a_cur[MT];
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) a_cur[mt] = wr[mt * TN];
+                        wr += (size_t)KL * P.Mp;
+                        __builtin_amdgcn_sched_barrier(0);
+                        const T v = sample<T, ND>(plane, lidx, t.f);
+                        const T b = (near && s * KL + q < nch) ? v : (T)0;
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a_cur[mt], b, acc[mt]);
+                        plane += KL * P.hstride;
+                    }
+                } else {
                     const T* plane = sIn;
                     const T* wr = wrow;
                     T a_next[MT];
@@ -421,9 +440,8 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
                         wr += (size_t)KL * P.Mp;                           // rows past the chunk stay inside the padded weight
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt) a_next[mt] = wr[mt * TN];
-                        // (few accumulators: the compiler otherwise moves these loads behind the
-                        // first MFMA of the step, where they are waited for at once; pinned at the end
-                        // of the step they stay here and have the whole step to arrive)
+                        // (few accumulators: here too the loads are kept above the step's arithmetic,
+                        // and pinned at its end they are first waited for there)
                         if constexpr (MT <= 2) __builtin_amdgcn_sched_barrier(0);
                         const T v = sample<T, ND>(plane, lidx, t.f);
                         const T b = (near && s * KL + q < nch) ? v : (T)0;
