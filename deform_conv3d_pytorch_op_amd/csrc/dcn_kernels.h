@@ -394,11 +394,11 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
                 // the next tap's offsets travel while this tap is computed
                 if (tap + 1 < P.kV) load_offsets<T, ND>(P, off_dg + (size_t)(tap + 1) * ND * P.outV, pos, onext);
                 TapGeo<T, ND> t;
-                tap_setup<T, ND>(P, ocur, ib, kd, t);
+                tap_setup_noidx<T, ND>(P, ocur, ib, kd, t);
                 const bool live = valid && t.inside;
                 if (!__any(live)) continue;        // whole wave outside: these column rows are zero
                 unsigned lidx[NC];
-                const bool in_halo = halo_corners<T, ND>(P, tg.hb, t, lidx);
+                const bool in_halo = halo_corners_strided<T, ND>(P, tg.hb, t, lidx);
                 const bool near = live && in_halo;                         // sampled from LDS
                 const bool far = live && !in_halo;                         // sampled from global memory
 #pragma unroll
@@ -455,6 +455,7 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
                     }
                 }
                 if (__any(far)) {                  // rare: some sample of this wave reaches past the halo
+                    tap_corner_idx<T, ND>(P, t);
                     unsigned voff[NC];
 #pragma unroll
                     for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
