@@ -383,11 +383,19 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
             const int nsteps = (nch + KL - 1) / KL;
             T onext[ND];
             load_offsets<T, ND>(P, off_dg, pos, onext);                    // offsets of tap 0
+
+            int kk[ND];                                                    // tap coordinates, counted up with the tap (no divisions)
+#pragma unroll
+            for (int a = 0; a < ND; ++a) kk[a] = 0;
             for (int tap = 0; tap < P.kV; ++tap) {
-                int kk[ND], kd[ND];
-                decode_tap<ND>(P, tap, kk);
+                int kd[ND];
 #pragma unroll
                 for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+#pragma unroll
+                for (int a = ND - 1; a >= 0; --a) {                        // next tap: increment with carry, fastest axis last
+                    if (++kk[a] < P.k[slot<ND>(a)] || a == 0) break;
+                    kk[a] = 0;
+                }
                 T ocur[ND];
 #pragma unroll
                 for (int a = 0; a < ND; ++a) ocur[a] = onext[a];
