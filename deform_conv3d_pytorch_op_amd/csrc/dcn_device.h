@@ -189,6 +189,29 @@ __device__ inline void tap_setup_noidx(const Params& P, const T offv[ND], const 
     }
     t.inside = inside;
 }
+// Corner offsets in units of `unit` (voxel index * unit), all zero unless `ok`: the low corner's
+// offset from three integer multiplies, the other corners by adding the strides of the axes whose
+// high corner has not collapsed onto the low one (a multiply per corner costs four times an add).
+template <typename T, int ND>
+__device__ inline void tap_corner_offsets(const Params& P, const TapGeo<T, ND>& t, bool ok, unsigned unit,
+                                          unsigned o[1 << ND]) {
+    if constexpr (ND == 3) {
+        const unsigned u2 = unit, u1 = (unsigned)P.in[2] * unit, u0 = (unsigned)P.in[1] * u1;       // uniform
+        const unsigned base = (((unsigned)t.lo[0] * (unsigned)P.in[1] + (unsigned)t.lo[1]) * (unsigned)P.in[2] + (unsigned)t.lo[2]) * unit;
+        const unsigned b = ok ? base : 0u;
+        const unsigned s0 = (ok && t.hi[0] != t.lo[0]) ? u0 : 0u, s1 = (ok && t.hi[1] != t.lo[1]) ? u1 : 0u;
+        const unsigned s2 = (ok && t.hi[2] != t.lo[2]) ? u2 : 0u;
+        o[0] = b;      o[1] = b + s2;      o[2] = b + s1;      o[3] = b + s1 + s2;
+        o[4] = b + s0; o[5] = b + s0 + s2; o[6] = b + s0 + s1; o[7] = b + s0 + s1 + s2;
+    } else {
+        const unsigned u1 = unit, u0 = (unsigned)P.in[2] * unit;
+        const unsigned base = ((unsigned)t.lo[0] * (unsigned)P.in[2] + (unsigned)t.lo[1]) * unit;
+        const unsigned b = ok ? base : 0u;
+        const unsigned s0 = (ok && t.hi[0] != t.lo[0]) ? u0 : 0u, s1 = (ok && t.hi[1] != t.lo[1]) ? u1 : 0u;
+        o[0] = b; o[1] = b + s1; o[2] = b + s0; o[3] = b + s0 + s1;
+    }
+}
+
 template <typename T, int ND>
 __device__ inline void tap_corner_idx(const Params& P, TapGeo<T, ND>& t) {
     if constexpr (ND == 3) {

@@ -1369,7 +1369,11 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 #pragma unroll
         for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
         TapGeo<T, ND> t;
-        tap_setup<T, ND>(P, off + (((size_t)n * P.DG + dg) * P.kV + tap) * ND * P.outV, posc, ib, kd, t);
+        {
+            T offv[ND];
+            load_offsets<T, ND>(P, off + (((size_t)n * P.DG + dg) * P.kV + tap) * ND * P.outV, posc, offv);
+            tap_setup_noidx<T, ND>(P, offv, ib, kd, t);
+        }
         const bool live = valid && t.inside;
 
         // LDS operations of one wavefront execute in order; the fences only pin the compiler
@@ -1385,8 +1389,10 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
                 const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
                 cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
             }
+            unsigned cb[NC];
+            tap_corner_offsets<T, ND>(P, t, live, cinB, cb);
 #pragma unroll
-            for (int i = 0; i < NC; ++i) sIdx[wave][j][i] = live ? t.idx[i] * cinB : 0u;
+            for (int i = 0; i < NC; ++i) sIdx[wave][j][i] = cb[i];
 #pragma unroll
             for (int i = 0; i < NC; ++i) sCw[wave][j][i] = live ? cw[i] : (T)0;
             sLive[wave][j] = live ? 1u : 0u;
