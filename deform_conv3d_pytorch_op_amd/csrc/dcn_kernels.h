@@ -917,21 +917,14 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         const T* gbase = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV;
         const unsigned b_off = (unsigned)q * P.outV + pos;
         const size_t gstep = (size_t)KL * P.outV;
-        // Reduction step k of this lane.  Rows past M read row 0 of the same position instead (the
-        // weight rows they meet are zero padding) and lanes outside the volume read a clamped
-        // position (their columns are never used), so the load itself needs no mask; `masked`
-        // additionally zeroes both cases for the bound below.
-        auto load_b = [&](int k, bool masked) -> T {
-            const int row0 = k * KL;                // uniform
-            const bool ok = row0 + q < P.M;
-            const T* gb = gbase + (size_t)(row0 < P.M ? k : 0) * gstep;
-            const T b = gb[ok ? b_off : pos];
-            return (!masked || (ok && valid)) ? b : (T)0;
-        };
-        // The same operand for the batches of the GEMM loops: the row base advances in scalar
-        // registers, clamped at the last real step (further steps of a batch meet zero weight rows
-        // and re-read that step), and the lane adds a 32-bit byte offset, so that a load costs a
-        // few scalar instructions and one select instead of 64-bit address arithmetic per lane.
+        // Reduction step k of this lane reads grad_output[k * KL + q][pos]: the row base advances in
+        // scalar registers, clamped at the last real step (the further steps of a batch meet zero
+        // weight rows and re-read that step; a lane whose row of the last step lies past M reads
+        // row q = 0 of it, again against a zero weight row), and the lane adds a 32-bit byte
+        // offset, so that a load costs a few scalar instructions and one select instead of 64-bit
+        // address arithmetic per lane.  Lanes outside the volume read a clamped position (their
+        // columns are never used).  No load is masked: a masked load becomes a conditional one,
+        // issued alone with a full wait behind it.
         const int klast = (P.M + KL - 1) / KL - 1;
         const unsigned b_byte = b_off * (unsigned)sizeof(T);
         const unsigned b_byte_last = (klast * KL + q < P.M ? b_off : pos) * (unsigned)sizeof(T);
