@@ -46,6 +46,9 @@ def load():
             f.restype, f.argtypes = _c_int, [_c_vp] * 6 + geom + tail
             f = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
             f.restype, f.argtypes = _c_int, [_c_vp] * 4 + geom + tail
+            if nd == 3:
+                f = getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)
+                f.restype, f.argtypes = _c_int, [_c_vp] * 6 + geom + tail + [ctypes.c_uint]
     if L.dcn_version() != 1:
         raise ImportError("libdcn_amd.so has ABI version %d, expected 1" % L.dcn_version())
     _lib = L
@@ -59,4 +62,6 @@ def check(rc):
 
 EXPORTS = ["dcn_version", "dcn_arch", "dcn_last_error", "dcn_workspace_bytes"] + [
     "dcn%dd_%s_%s" % (nd, op, suf)
-    for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight") for suf in ("f32", "f64")]
+    for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight") for suf in ("f32", "f64")] + [
+    "dcn3d_backward_input_offset_flags_f32", "dcn3d_backward_input_offset_flags_f64"]
+FLAG_OOB_OFFSET_GRAD_ZERO = 1

@@ -118,6 +118,7 @@ int validate(const Geometry& g, Params& P) {
     // channels-last voxel*channel offsets of one sample are 32-bit as well
     if (inV * g.C_in > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one input sample exceeds 2^31 elements");
     if (g.N > 65535) return fail(DCN_E_ARGUMENT, "batch exceeds 65535");
+    P.oob_zero = 0;
     P.nd = g.nd; P.N = g.N; P.C_in = g.C_in; P.C_out = g.C_out; P.G = g.G; P.cpg = g.cpg; P.DG = g.C_in / g.cpg;
     P.M = g.C_out / g.G; P.Cg = g.C_in / g.G;
     for (int a = 0; a < 3; ++a) {
@@ -349,9 +350,11 @@ int absmax(const T* w, size_t n, float* out, hipStream_t s) {
 
 template <typename T, int ND>
 int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* off, const T* gout, T* gin,
-                          T* goff, void* ws, size_t ws_bytes, hipStream_t s) {
+                          T* goff, void* ws, size_t ws_bytes, hipStream_t s, unsigned flags = 0) {
     Params P;
     if (int rc = validate(g, P)) return rc;
+    if (flags & ~(unsigned)DCN_FLAG_OOB_OFFSET_GRAD_ZERO) return fail(DCN_E_ARGUMENT, "unknown flag");
+    P.oob_zero = (flags & DCN_FLAG_OOB_OFFSET_GRAD_ZERO) ? 1 : 0;
     if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     bwd_data_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
     const size_t wbytes = bwd_data_weight_bytes<T>(P.M, P.Cg, P.kV, P.G);
@@ -657,6 +660,14 @@ size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, 
         return backward_input_offset<T, 3>(geo3(G3_ARGS), input, weight, offset, grad_output, grad_input,           \
                                            grad_offset, workspace, workspace_bytes,                                 \
                                            static_cast<hipStream_t>(stream));                                       \
+    }                                                                                                               \
+    int dcn3d_backward_input_offset_flags_##SUF(const T* input, const T* weight, const T* offset,                   \
+                                                const T* grad_output, T* grad_input, T* grad_offset,                \
+                                                DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes,            \
+                                                void* stream, unsigned flags) {                                     \
+        return backward_input_offset<T, 3>(geo3(G3_ARGS), input, weight, offset, grad_output, grad_input,           \
+                                           grad_offset, workspace, workspace_bytes,                                 \
+                                           static_cast<hipStream_t>(stream), flags);                                \
     }                                                                                                               \
     int dcn3d_backward_weight_##SUF(const T* input, const T* offset, const T* grad_output, T* grad_weight,          \
                                     DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {        \

@@ -31,6 +31,7 @@ struct Params {
     int hvol;                     // hext[0] * hext[1] * hext[2]
     int hstride;                  // LDS elements between the planes of two channels (>= hvol)
     int cchunk;                   // channels staged per pass
+    int oob_zero;                 // 3-D backward: 1 = no grad_offset term for out-of-range samples
 };
 
 // ---------------------------------------------------------------------------------------------

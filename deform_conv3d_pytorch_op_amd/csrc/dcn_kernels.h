@@ -648,7 +648,7 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
         tap_setup<T, ND>(P, ocur, ib, kd, t);
         const bool live = valid && t.inside;
         T oob[3] = {0, 0, 0};
-        if (ND == 3 && valid && !t.inside) {
+        if (ND == 3 && valid && !t.inside && !P.oob_zero) {
             const T len = (T)P.in[0];
 #pragma unroll
             for (int a = 0; a < ND; ++a) oob[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= len) ? (T)1 : (T)0);
@@ -1132,7 +1132,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     for (int i = 0; i < NC; ++i) cwd[i] = (double)cw[i];
                     // out-of-range samples of the 3-D operator: +-|gcol| per axis; h and w are compared
                     // with the LENGTH extent
-                    const bool oor = COORD && ND == 3 && slot_ok && !t.inside;
+                    const bool oor = COORD && ND == 3 && slot_ok && !t.inside && !P.oob_zero;
                     T sg[ND];
 #pragma unroll
                     for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= (T)P.in[0]) ? (T)1 : (T)0);

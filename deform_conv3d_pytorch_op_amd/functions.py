@@ -5,8 +5,11 @@ deform2d/deform_conv2d_functions/deform_conv2d_function.py:7-57 is its float, di
 group-1, bias-free subset).
 
 Same call shape: `Fn.apply(inputs, offset, weight, bias=None, stride, padding, dilation,
-channel_per_group=1, group=1)` (plus one optional trailing argument, `standard_output_size`, see
-`output_size`); same dilation-blind output size by default; same shape checks and messages
+channel_per_group=1, group=1)` (plus two optional trailing arguments: `standard_output_size`, see
+`output_size`, and `oob_offset_grad`: 'reference' keeps the 3-D kernels' +-|grad column| term in
+grad_offset for samples outside the input (deform3d/lib/deform_conv3d_cuda_kernel.cu:470-481), 'zero'
+leaves it out, which makes grad_offset the derivative of the forward pass everywhere); same
+dilation-blind output size by default; same shape checks and messages
 as the reference's `shape_check` (deform3d/lib/deform_conv3d_cuda.cpp:24-87), raised as
 RuntimeError.  Differences: no column workspace is kept on ctx (the kernels never build one),
 float32 and float64 are served by the same class for both 2-D and 3-D, and gradients that are
@@ -137,7 +140,7 @@ def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channe
 
 
 def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation, channel_per_group, group,
-              need_data, need_weight, standard=False):
+              need_data, need_weight, standard=False, oob_zero=False):
     L = _lib.load()
     _device_check(inputs, offset, weight, grad_output)
     outs = tuple(grad_output.shape[2:])
@@ -155,9 +158,12 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
             # every element of grad_offset
             grad_input = torch.zeros_like(inputs)
             grad_offset = torch.empty_like(offset)
-            fn = getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))
-            _lib.check(fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
-                          grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, _stream()))
+            args = (inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
+                    grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, _stream())
+            if nd == 3 and oob_zero:        # the reference's 2-D kernels have no out-of-range term
+                _lib.check(getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)(*args, _lib.FLAG_OOB_OFFSET_GRAD_ZERO))
+            else:
+                _lib.check(getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))(*args))
         if need_weight:
             grad_weight = torch.zeros_like(weight)          # beta = 1 accumulation, as in the reference
             fn = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
@@ -171,9 +177,12 @@ class _ConvOffsetNdFunction(Function):
 
     @classmethod
     def _fwd(cls, ctx, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group,
-             standard_output_size=False):
+             standard_output_size=False, oob_offset_grad="reference"):
         nd = cls.ND
         ctx.standard = bool(standard_output_size)
+        if oob_offset_grad not in ("reference", "zero"):
+            raise ValueError("oob_offset_grad must be 'reference' or 'zero'")
+        ctx.oob_zero = oob_offset_grad == "zero"
         ctx.stride, ctx.padding, ctx.dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
         ctx.channel_per_group, ctx.group = int(channel_per_group), int(group)
         ctx.has_bias = bias is not None
@@ -187,11 +196,12 @@ class _ConvOffsetNdFunction(Function):
         need = ctx.needs_input_grad
         # grad_input and grad_offset come out of one kernel, as in the reference (:52)
         gi, go, gw = _backward(cls.ND, inputs, offset, weight, grad_output, ctx.stride, ctx.padding, ctx.dilation,
-                               ctx.channel_per_group, ctx.group, need[0] or need[1], need[2], ctx.standard)
+                               ctx.channel_per_group, ctx.group, need[0] or need[1], need[2], ctx.standard,
+                               ctx.oob_zero)
         gb = None
         if ctx.has_bias and need[3]:
             gb = grad_output.sum(dim=[0] + list(range(2, 2 + cls.ND)))
-        return (gi if need[0] else None, go if need[1] else None, gw, gb, None, None, None, None, None, None)
+        return (gi if need[0] else None, go if need[1] else None, gw, gb, None, None, None, None, None, None, None)
 
 
 class ConvOffset3dFunction(_ConvOffsetNdFunction):
@@ -199,9 +209,9 @@ class ConvOffset3dFunction(_ConvOffsetNdFunction):
 
     @staticmethod
     def forward(ctx, inputs, offset, weight, bias=None, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1),
-                channel_per_group=1, group=1, standard_output_size=False):
+                channel_per_group=1, group=1, standard_output_size=False, oob_offset_grad="reference"):
         return ConvOffset3dFunction._fwd(ctx, inputs, offset, weight, bias, stride, padding, dilation,
-                                         channel_per_group, group, standard_output_size)
+                                         channel_per_group, group, standard_output_size, oob_offset_grad)
 
     @staticmethod
     @once_differentiable
@@ -214,9 +224,9 @@ class ConvOffset2dFunction(_ConvOffsetNdFunction):
 
     @staticmethod
     def forward(ctx, inputs, offset, weight, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
-                channel_per_group=1, group=1, standard_output_size=False):
+                channel_per_group=1, group=1, standard_output_size=False, oob_offset_grad="reference"):
         return ConvOffset2dFunction._fwd(ctx, inputs, offset, weight, bias, stride, padding, dilation,
-                                         channel_per_group, group, standard_output_size)
+                                         channel_per_group, group, standard_output_size, oob_offset_grad)
 
     @staticmethod
     @once_differentiable

@@ -13,8 +13,9 @@ Initialisation: the reference draws Kaiming-normal (fan_out) and then overwrites
 the constant 1 (deform_conv3d_model.py:38-39); this keeps the Kaiming draw, which is what the
 float 2-D package does (deform2d ... :29).  Bias ~ U(-0.1, 0.1) as in the reference (:42).
 `device` and `dtype` are extra keyword arguments (the reference hard-codes cuda float / double),
-and so is `standard_output_size` (default False: the reference's dilation-blind output size; True:
-the usual dilation-aware one, see functions.output_size).
+and so are `standard_output_size` (default False: the reference's dilation-blind output size; True:
+the usual dilation-aware one, see functions.output_size) and `oob_offset_grad` (default 'reference';
+'zero' drops the 3-D kernels' grad_offset term for samples outside the input, see functions.py).
 
 `ConvOffset{2,3}dPack` additionally own the plain convolution that the reference's callers put in
 front of the layer to produce the offsets (deform3d/test_model.py:18-30, deform2d/test_model.py:19-29):
@@ -33,9 +34,13 @@ class _ConvOffsetNd(nn.Module):
     _function = None
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
-                 channel_per_group=1, bias=True, groups=1, device=None, dtype=None, standard_output_size=False):
+                 channel_per_group=1, bias=True, groups=1, device=None, dtype=None, standard_output_size=False,
+                 oob_offset_grad="reference"):
         super().__init__()
         self.standard_output_size = bool(standard_output_size)
+        if oob_offset_grad not in ("reference", "zero"):
+            raise ValueError("oob_offset_grad must be 'reference' or 'zero'")
+        self.oob_offset_grad = oob_offset_grad
         self.in_channels = in_channels
         self.out_channels = out_channels
         self.kernel_size = self._tuple(kernel_size)
@@ -59,7 +64,8 @@ class _ConvOffsetNd(nn.Module):
 
     def forward(self, input, offset):
         return self._function.apply(input, offset, self.weight, self.bias, self.stride, self.padding,
-                                    self.dilation, self.channel_per_group, self.group, self.standard_output_size)
+                                    self.dilation, self.channel_per_group, self.group, self.standard_output_size,
+                                    self.oob_offset_grad)
 
     def extra_repr(self):
         return ('{in_channels}, {out_channels}, kernel_size={kernel_size}, stride={stride}, padding={padding}, '
@@ -80,9 +86,10 @@ class _ConvOffsetPackNd(_ConvOffsetNd):
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
                  channel_per_group=1, bias=True, groups=1, zero_init_offset=False, device=None, dtype=None,
-                 standard_output_size=False):
+                 standard_output_size=False, oob_offset_grad="reference"):
         super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, channel_per_group,
-                         bias, groups, device=device, dtype=dtype, standard_output_size=standard_output_size)
+                         bias, groups, device=device, dtype=dtype, standard_output_size=standard_output_size,
+                         oob_offset_grad=oob_offset_grad)
         if in_channels % channel_per_group != 0:
             raise ValueError('in_channels must be divisible by channel_per_group')
         taps = 1

@@ -91,6 +91,22 @@ int dcn3d_backward_input_offset_f64(const double *input, const double *weight, c
                                     const double *grad_output, double *grad_input, double *grad_offset,
                                     DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same call with option flags.  No counterpart in the reference, whose 3-D col2im_offset kernel
+ * always adds +-|grad column| to grad_offset for a sample that lies outside the input
+ * (deform3d/lib/deform_conv3d_cuda_kernel.cu:470-481), although such a sample contributes nothing to
+ * the output: with DCN_FLAG_OOB_OFFSET_GRAD_ZERO that term is left out and grad_offset is the
+ * derivative of the forward pass everywhere.  flags = 0 is dcn3d_backward_input_offset_*; other
+ * bits are rejected.  (The reference's 2-D kernels have no such term.) */
+#define DCN_FLAG_OOB_OFFSET_GRAD_ZERO 1u
+int dcn3d_backward_input_offset_flags_f32(const float *input, const float *weight, const float *offset,
+                                          const float *grad_output, float *grad_input, float *grad_offset,
+                                          DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes,
+                                          void *stream, unsigned flags);
+int dcn3d_backward_input_offset_flags_f64(const double *input, const double *weight, const double *offset,
+                                          const double *grad_output, double *grad_input, double *grad_offset,
+                                          DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes,
+                                          void *stream, unsigned flags);
+
 int dcn3d_backward_weight_f32(const float *input, const float *offset, const float *grad_output,
                               float *grad_weight, DCN3D_GEOMETRY, void *workspace,
                               size_t workspace_bytes, void *stream);

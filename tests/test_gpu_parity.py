@@ -144,6 +144,71 @@ def test_gradcheck_3d_float64_in_range():
                                     eps=1e-6, atol=1e-5, rtol=1e-3, nondet_tol=1e-9)
 
 
+def _inside_mask(c):
+    """[N, DG, kV, outV] bool: the sample of (deformable group, tap, position) lies inside the input
+    (-1 < coordinate < size on every axis), worked out here from the offsets in float64."""
+    nd = c["nd"]
+    N = c["x"].shape[0]
+    kV, outV = math.prod(c["k"]), math.prod(c["outs"])
+    off = c["off"].double().reshape(N, -1, kV, nd, outV)
+    grids = torch.meshgrid(*[torch.arange(o, dtype=torch.float64) for o in c["outs"]], indexing="ij")
+    taps = torch.meshgrid(*[torch.arange(k, dtype=torch.float64) for k in c["k"]], indexing="ij")
+    ok = torch.ones(off.shape[0], off.shape[1], kV, outV, dtype=torch.bool)
+    for a in range(nd):
+        base = grids[a].reshape(1, 1, 1, outV) * c["stride"][a] - c["pad"][a]
+        tap = taps[a].reshape(1, 1, kV, 1) * c["dil"][a]
+        p = base + tap + off[:, :, :, a, :]
+        ok &= (p > -1) & (p < c["ins"][a])
+    return ok
+
+
+@pytest.mark.parametrize("name", ["3d_basic", "3d_dilation3", "3d_c5_like"])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32], ids=["f64", "f32"])
+def test_oob_offset_grad_zero_drops_only_the_out_of_range_term(name, dtype):
+    """oob_offset_grad='zero': grad_offset of a sample outside the input is exactly zero, that of a
+    sample inside is what the reference mode gives (which the oracle pins), and nothing else moves."""
+    dcn = _dcn()
+    c = make_case(*SMALL_CASES[name], dtype=dtype, seed=21)
+    inside = _inside_mask(c)
+    assert 0 < int((~inside).sum()) < inside.numel()          # the case has samples of both kinds
+    dev = torch.device("cuda:0")
+    res = {}
+    for mode in ("reference", "zero"):
+        x, off, w = (c[k].to(dev).requires_grad_(True) for k in ("x", "off", "w"))
+        out = dcn.ConvOffset3dFunction.apply(x, off, w, None, c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"],
+                                             False, mode)
+        out.backward(c["gout"].to(dev))
+        torch.cuda.synchronize()
+        res[mode] = (out.detach().cpu(), x.grad.cpu(), off.grad.cpu(), w.grad.cpu())
+    tol = TOL[dtype]["grad"]
+    assert torch.equal(res["zero"][0], res["reference"][0])
+    assert rel_err(res["zero"][1], res["reference"][1]) <= tol
+    assert rel_err(res["zero"][3], res["reference"][3]) <= tol
+    N, kV, nd, outV = c["x"].shape[0], math.prod(c["k"]), c["nd"], math.prod(c["outs"])
+    go_ref = res["reference"][2].reshape(N, -1, kV, nd, outV)
+    go_zero = res["zero"][2].reshape(N, -1, kV, nd, outV)
+    m = inside.unsqueeze(3).expand_as(go_ref)
+    assert torch.count_nonzero(go_zero[~m]) == 0
+    assert go_ref[~m].abs().max() > 0                           # the reference mode does put something there
+    scale = go_ref.abs().max().item()
+    assert (go_zero[m].double() - go_ref[m].double()).abs().max().item() <= tol * scale
+
+
+def test_gradcheck_3d_float64_oob_zero():
+    # with the out-of-range term left out grad_offset is a derivative everywhere, so gradcheck also
+    # passes with samples outside the volume (offsets up to 3 voxels on a 5^3 input, padding 1)
+    print("gradcheck 3d oob zero", flush=True)
+    dcn = _dcn()
+    g = torch.Generator().manual_seed(10)
+    dev = "cuda:0"
+    x = torch.randn(1, 2, 5, 5, 5, generator=g, dtype=torch.float64).to(dev).requires_grad_(True)
+    off = ((torch.rand(1, 48, 6, 6, 6, generator=g, dtype=torch.float64) * 2 - 1) * 3).to(dev).requires_grad_(True)
+    w = torch.randn(2, 1, 2, 2, 2, generator=g, dtype=torch.float64).to(dev).requires_grad_(True)
+    fn = lambda x_, o_, w_: dcn.ConvOffset3dFunction.apply(x_, o_, w_, None, (1, 1, 1), (1, 1, 1), (1, 1, 1), 1, 2,
+                                                           False, "zero")
+    assert torch.autograd.gradcheck(fn, (x, off, w), eps=1e-6, atol=1e-5, rtol=1e-3, nondet_tol=1e-9)
+
+
 def test_modules_forward_backward():
     print("modules", flush=True)
     dcn = _dcn()

@@ -166,3 +166,11 @@ def test_pack_module_offset_convolution_follows_output_size_mode():
     assert blind.conv_offset.dilation == (1, 1) and std.conv_offset.dilation == (2, 2)
     x = torch.zeros(1, 4, 9, 9)
     assert blind.conv_offset(x).shape[2:] == (11, 11) and std.conv_offset(x).shape[2:] == (9, 9)
+
+
+def test_oob_offset_grad_argument_is_validated():
+    from deform_conv3d_pytorch_op_amd import ConvOffset3d, ConvOffset3dPack
+    assert ConvOffset3d(2, 2, 3, oob_offset_grad="zero").oob_offset_grad == "zero"
+    assert ConvOffset3dPack(2, 2, 3).oob_offset_grad == "reference"
+    with pytest.raises(ValueError):
+        ConvOffset3d(2, 2, 3, oob_offset_grad="clean")
