@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     ("c4", "forward"): 0.524e9,
     ("c4", "backward_input_offset"): 1.992e9,
-    ("c4", "backward_weight"): 1.051e9,
+    ("c4", "backward_weight"): 1.211e9,
 }
 
 # name: (nd, N, C_in, C_out, in, k, stride, pad, dil, cpg, groups, offset scale / dist, dtype)
