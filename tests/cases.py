@@ -59,3 +59,23 @@ SMALL_CASES = {
     "3d_dilation3": (3, 1, 4, 4, (8, 8, 8), 3, 1, 3, 3, 2, 1, 2.5),          # dilation-blind output 12^3: many taps out of range
     "3d_short_length": (3, 1, 4, 4, (2, 8, 8), (1, 3, 3), 1, (0, 1, 1), 1, 4, 1, 4.0),  # D < H: out-of-range branch vs length extent
 }
+
+
+def random_spec(seed):
+    """A small random geometry (the SMALL_CASES tuple layout), reproducible from `seed`: odd channel
+    counts, every divisor as channels per deformable group, rectangular kernels, strides, pads and
+    dilations per axis."""
+    import random
+    r = random.Random(1000 + seed)
+    nd = r.choice((2, 3))
+    groups = r.choice((1, 1, 2, 3))
+    cg = r.randint(1, 12)
+    c_in = groups * cg
+    cpg = r.choice([d for d in range(1, c_in + 1) if c_in % d == 0])
+    c_out = groups * r.randint(1, 40 if nd == 2 else 24)
+    k = tuple(r.randint(1, 3) for _ in range(nd))
+    stride = tuple(r.randint(1, 2) for _ in range(nd))
+    dil = tuple(r.randint(1, 2) for _ in range(nd))
+    pad = tuple(r.randint(0, 2) for _ in range(nd))
+    ins = tuple(r.randint(max(3, kk - 2 * p), 12 if nd == 2 else 8) for kk, p in zip(k, pad))
+    return (nd, r.randint(1, 3), c_in, c_out, ins, k, stride, pad, dil, cpg, groups, r.choice((0.5, 2.0, 4.0)))

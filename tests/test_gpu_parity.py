@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import dcn_oracle as orc
-from tests.cases import SMALL_CASES, make_case
+from tests.cases import SMALL_CASES, make_case, random_spec
 
 pytestmark = pytest.mark.gpu
 
@@ -68,6 +68,16 @@ def test_small_cases_match_oracle(name, dtype):
     print("case", name, dtype, flush=True)
     c = make_case(*SMALL_CASES[name], dtype=dtype, seed=3)
     compare(c, dtype, name)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_geometries_match_oracle(seed):
+    """Seeded random small geometries (2-D / 3-D, odd channel counts, all divisors as deformable-group
+    widths, rectangular kernels, per-axis stride / padding / dilation), float64 and float32."""
+    spec = random_spec(seed)
+    print("random geometry", seed, spec, flush=True)
+    for dtype in (torch.float64, torch.float32):
+        compare(make_case(*spec, dtype=dtype, seed=100 + seed), dtype, "random_%d" % seed)
 
 
 @pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz"))),
