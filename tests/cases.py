@@ -61,15 +61,15 @@ SMALL_CASES = {
 }
 
 
-def random_spec(seed):
+def random_spec(seed, medium=False):
     """A small random geometry (the SMALL_CASES tuple layout), reproducible from `seed`: odd channel
     counts, every divisor as channels per deformable group, rectangular kernels, strides, pads and
-    dilations per axis."""
+    dilations per axis.  `medium`: extents of several position tiles per axis and more channels."""
     import random
-    r = random.Random(1000 + seed)
+    r = random.Random((5000 if medium else 1000) + seed)
     nd = r.choice((2, 3))
     groups = r.choice((1, 1, 2, 3))
-    cg = r.randint(1, 12)
+    cg = r.randint(1, 12) if not medium else r.randint(4, 24)
     c_in = groups * cg
     cpg = r.choice([d for d in range(1, c_in + 1) if c_in % d == 0])
     c_out = groups * r.randint(1, 40 if nd == 2 else 24)
@@ -77,5 +77,8 @@ def random_spec(seed):
     stride = tuple(r.randint(1, 2) for _ in range(nd))
     dil = tuple(r.randint(1, 2) for _ in range(nd))
     pad = tuple(r.randint(0, 2) for _ in range(nd))
+    if medium:
+        ins = tuple(r.randint(14, 40 if nd == 2 else 20) for _ in range(nd))
+        return (nd, r.randint(1, 2), c_in, c_out, ins, k, stride, pad, dil, cpg, groups, r.choice((0.5, 1.5, 3.0)))
     ins = tuple(r.randint(max(3, kk - 2 * p), 12 if nd == 2 else 8) for kk, p in zip(k, pad))
     return (nd, r.randint(1, 3), c_in, c_out, ins, k, stride, pad, dil, cpg, groups, r.choice((0.5, 2.0, 4.0)))

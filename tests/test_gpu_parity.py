@@ -80,6 +80,16 @@ def test_random_geometries_match_oracle(seed):
         compare(make_case(*spec, dtype=dtype, seed=100 + seed), dtype, "random_%d" % seed)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_medium_geometries_match_oracle(seed):
+    """The same with extents of several position tiles per axis (halo tiling, channel splits, partial
+    tiles at the rim) and up to 72 input channels."""
+    spec = random_spec(seed, medium=True)
+    print("random medium geometry", seed, spec, flush=True)
+    for dtype in (torch.float64, torch.float32):
+        compare(make_case(*spec, dtype=dtype, seed=200 + seed), dtype, "random_medium_%d" % seed)
+
+
 @pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz"))),
                          ids=lambda p: os.path.basename(p)[:-4])
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32], ids=["f64", "f32"])
