@@ -1021,6 +1021,30 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             auto gemm_tail = [&](typename MM::Acc& dd, const T* wp, int k_begin) {
                 T a_nx[AB], b_nx[AB];
                 load_batch(a_nx, b_nx, wp, k_begin);
+                if (PACKW && ksteps - k_begin >= 96) {
+                    // Long reductions (M >= 192 float): the next batch is requested in the same block
+                    // as this batch's MFMAs (past the last step the padded slab's last batch is read
+                    // again) and the scheduler is told to deal the address arithmetic and the loads out
+                    // between the MFMAs.  The wavefronts of a workgroup run in step, so a separate load
+                    // phase leaves the matrix pipe idle in all of them at once.  (Short reductions lose
+                    // more to the one redundant batch than they gain.)
+                    for (int k0 = k_begin; k0 < ksteps; k0 += AB) {
+                        T a_cu[AB], b_cu[AB];
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) { a_cu[k] = a_nx[k]; b_cu[k] = b_nx[k]; }
+                        load_batch(a_nx, b_nx, wp, min(k0 + AB, (int)(wpass / 64) - AB));
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_cu[k], b_cu[k], dd);
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x004, 12, 0);     // scalar address arithmetic
+                            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);      // vector
+                            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);      // two loads
+                        }
+                    }
+                    return;
+                }
                 for (int k0 = k_begin; k0 < ksteps; k0 += AB) {
                     T a_cu[AB], b_cu[AB];
 #pragma unroll

@@ -46,6 +46,7 @@ SMALL_CASES = {
     "2d_many_m_chunks": (2, 1, 6, 300, (6, 7), 3, 1, 1, 1, 6, 1, 1.0),     # M > 8 row tiles of 32
     "2d_c3_like": (2, 1, 16, 8, 10, 3, 1, 2, 2, 4, 2, 3.0),                # groups 2, 4 deformable groups, dilation 2
     "2d_cpg_straddles_groups": (2, 1, 12, 4, 6, 3, 1, 1, 1, 12, 2, 1.5),   # one deformable group over two conv groups
+    "2d_long_reduction": (2, 1, 8, 400, (6, 7), 3, 1, 1, 1, 8, 1, 1.0),           # M = 400: the long-reduction form of the fused kernel's GEMM loop in both precisions
     "2d_chunk8_ragged": (2, 2, 22, 10, (9, 8), 3, 1, 1, 1, 11, 1, 2.0),            # 11-channel segments: chunks of 8 + 3
     "2d_cpg_unaligned": (2, 1, 12, 6, 6, 2, 1, 0, 1, 4, 2, 1.5),           # cpg 4, 6 channels per conv group
     "3d_basic": (3, 2, 4, 4, (5, 6, 7), 3, 1, 1, 1, 2, 2, 3.0),
