@@ -196,6 +196,10 @@ static int fused_first_waves() {
     static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : 8; }();
     return v;
 }
+static bool fused_fixed_stride() {      // DCN_FUSED_FIXED=0: runtime plane stride even where the compile-time one fits
+    static const int v = [] { const char* e = getenv("DCN_FUSED_FIXED"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
+}
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
     return v != 0;
@@ -378,7 +382,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         Params Ph = P;
         if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T), nw, nw != 8)) continue;
         const size_t tables = (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
-        const bool fixed = Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
+        const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
         if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
         if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) < 4) continue;
         // Channels per chunk: 8 where that takes fewer MFMA passes per channel (a pass holds TN / CCH

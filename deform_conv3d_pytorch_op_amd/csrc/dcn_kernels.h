@@ -114,7 +114,8 @@ __global__ __launch_bounds__(WG) void forward_kernel(Params P, const T* __restri
             TapGeo<T, ND> t;
             tap_setup<T, ND>(P, off_dg + (size_t)tap * ND * P.outV, posc, ib, kd, t);
             const bool live = valid && t.inside;
-            if (!__any(live)) continue;        // whole wave outside: the column rows are zero
+            // (a wave whose samples are all outside still multiplies its zero column rows: with a
+            // non-finite weight the reference's GEMM turns them into NaN, and so does this)
             unsigned voff[NC];
 #pragma unroll
             for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
@@ -404,7 +405,8 @@ __global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T
                 TapGeo<T, ND> t;
                 tap_setup_noidx<T, ND>(P, ocur, ib, kd, t);
                 const bool live = valid && t.inside;
-                if (!__any(live)) continue;        // whole wave outside: these column rows are zero
+                // (a wave whose samples are all outside still multiplies its zero column rows: with a
+                // non-finite weight the reference's GEMM turns them into NaN, and so does this)
                 unsigned lidx[NC];
                 const bool in_halo = halo_corners_strided<T, ND>(P, tg.hb, t, lidx);
                 const bool near = live && in_halo;                         // sampled from LDS
@@ -749,7 +751,8 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
                             } else if constexpr (ND == 3) {
                                 const T av = gv > 0 ? gv : -gv;
 #pragma unroll
-                                for (int a = 0; a < ND; ++a) ga[r][a] += misc[3 + a] * av;
+                                for (int a = 0; a < ND; ++a)      // selected, not multiplied: 0 * inf would be NaN where the reference adds nothing
+                                    ga[r][a] += misc[3 + a] < (T)0 ? -av : (misc[3 + a] > (T)0 ? av : (T)0);
                             }
                         }
                     }
@@ -780,20 +783,27 @@ __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __
 // of magnitude slower than LDS integer atomics on gfx950, so float contributions are summed as
 // 64-bit fixed point: value * 2^e rounded to an integer and added with ds_add_u64.  The exponent
 // e is chosen per workgroup and convolution group from a bound on the largest possible term
-// (8 * max|W| * max_pos sum_m |grad_output|), leaving 2^16 terms of headroom below 2^51; the
-// integer sum is exact, so the result is rounded once when the cell is flushed.  double keeps a
+// (8 * max|W| * max_pos sum_m |grad_output|), leaving 2^17 terms of headroom below 2^47; the
+// integer sum is exact, so the result is rounded once when the cell is flushed.  A bound that is
+// not finite (NaN or infinity in grad_output or the weights) has no exponent: such a workgroup
+// sends every contribution through the global float atomics of the far path instead, which
+// propagate NaN and infinity like the reference's atomicAdd.  double keeps a
 // floating cell (ds_add_f64): its 1e-10 tolerance is tighter than the fixed-point grid.
 template <typename T> struct LdsCell;
 template <> struct LdsCell<float> {
     typedef unsigned long long type;
     static constexpr double MAGIC = 6755399441055744.0;     // 1.5 * 2^52: low mantissa bits = integer value
+    // The bit pattern of MAGIC + x is the pattern of MAGIC plus the integer x (|x| < 2^51), and the
+    // pattern of MAGIC is zero in its low 48 bits: the raw patterns are summed and, whatever the
+    // number of terms a cell receives, its low 48 bits hold the sum of the integers modulo 2^48.
     __device__ static inline void add(type* p, double w, double gv_scaled) {
         const double d = __builtin_fma(w, gv_scaled, MAGIC);
-        const long long bits = __double_as_longlong(d) - __double_as_longlong(MAGIC);
-        (void)__hip_atomic_fetch_add(p, (type)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        (void)__hip_atomic_fetch_add(p, (type)__double_as_longlong(d), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     __device__ static inline double pre(float gv, double scale) { return (double)gv * scale; }
-    __device__ static inline float value(type c, double inv_scale) { return (float)((double)(long long)c * inv_scale); }
+    __device__ static inline float value(type c, double inv_scale) {
+        return (float)((double)((long long)(c << 16) >> 16) * inv_scale);      // sign-extended low 48 bits
+    }
 };
 template <> struct LdsCell<double> {
     typedef double type;
@@ -804,22 +814,24 @@ template <> struct LdsCell<double> {
     __device__ static inline double value(type c, double) { return c; }
 };
 
-// max |w| over a small tensor (used for the fixed-point exponent).  Each workgroup reduces a
-// strided share and joins the result with an integer atomic max: non-negative floats order like
-// their bit patterns.  `out` must hold 0 beforehand.
+// max |w| over a small tensor (used for the fixed-point exponent), NaN if any element is NaN.  Each
+// workgroup reduces a strided share and joins the result with an integer atomic max: non-negative
+// floats order like their bit patterns.  `out` must hold 0 beforehand.
 template <typename T>
 __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restrict__ out) {
     __shared__ float red[256];
-    float m = 0.f;
+    // maxima are taken on the bit patterns: |NaN| has the largest pattern, so a NaN survives (fmaxf drops it)
+    unsigned m = 0u;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        m = fmaxf(m, fabsf((float)w[i]));
-    red[threadIdx.x] = m;
+        m = max(m, __float_as_uint(fabsf((float)w[i])));
+    unsigned* redu = reinterpret_cast<unsigned*>(red);
+    redu[threadIdx.x] = m;
     __syncthreads();
     for (int sft = blockDim.x / 2; sft > 0; sft >>= 1) {
-        if ((int)threadIdx.x < sft) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + sft]);
+        if ((int)threadIdx.x < sft) redu[threadIdx.x] = max(redu[threadIdx.x], redu[threadIdx.x + sft]);
         __syncthreads();
     }
-    if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned*>(out), __float_as_uint(red[0]));
+    if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned*>(out), redu[0]);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -968,18 +980,22 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         // 8 * max|W| * max_pos sum_m |grad_output|
 #pragma unroll
         for (int sh = TN; sh < 64; sh <<= 1) sabs += __shfl_xor(sabs, sh);
+        // maxima on the bit patterns (sabs >= 0 or NaN): a NaN has the largest pattern and survives
+        unsigned sbits = __float_as_uint(fabsf(sabs));
 #pragma unroll
-        for (int sh = 1; sh < TN; sh <<= 1) sabs = fmaxf(sabs, __shfl_xor(sabs, sh));
+        for (int sh = 1; sh < TN; sh <<= 1) sbits = max(sbits, (unsigned)__shfl_xor((int)sbits, sh));
         __syncthreads();
-        if (lane == 0) sRed[wave] = sabs;
+        if (lane == 0) sRed[wave] = __uint_as_float(sbits);
         __syncthreads();
-        float smax = 0.f;
+        unsigned smaxb = 0u;
 #pragma unroll
-        for (int w8 = 0; w8 < NW; ++w8) smax = fmaxf(smax, sRed[w8]);
+        for (int w8 = 0; w8 < NW; ++w8) smaxb = max(smaxb, __float_as_uint(sRed[w8]));
         int ex = 0;
-        const float bound = 8.f * wmax[0] * smax;
+        const float bound = 8.f * wmax[0] * __uint_as_float(smaxb);
+        // float cells need a finite bound; without one this workgroup scatters through the far path
+        const bool cells_ok = sizeof(T) == 8 || bound < 3.0e38f;      // false for NaN
         if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
-        const double scale = ldexp(1.0, 34 - ex), inv_scale = ldexp(1.0, ex - 34);
+        const double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
 
         for (int cc0 = rb; cc0 < re; cc0 += CCH) {
             if ((chunk_no++) % csplit != cz) continue;          // another workgroup's chunk (uniform)
@@ -1141,7 +1157,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     for (int a = 0; a < ND; ++a) ga[a] = 0;
                     // corner cells and weights, computed by every lane (dead lanes never use them)
                     unsigned lidx[NC];
-                    const bool in_halo = halo_corners_strided<T, ND>(P, tg.hb, t, lidx);
+                    const bool in_halo = halo_corners_strided<T, ND>(P, tg.hb, t, lidx) && cells_ok;
                     T cw[NC];
                     if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
                         const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
@@ -1227,7 +1243,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         } else if (oor) {
                             const T av = gv > 0 ? gv : -gv;
 #pragma unroll
-                            for (int a = 0; a < ND; ++a) ga[a] += sg[a] * av;
+                            for (int a = 0; a < ND; ++a)      // selected, not multiplied: 0 * inf would be NaN where the reference adds nothing
+                                ga[a] += sg[a] < (T)0 ? -av : (sg[a] > (T)0 ? av : (T)0);
                         }
                         // the next pass's MFMAs of this step, in uniform control flow
                         if (do_mma) {

@@ -134,6 +134,22 @@ def test_gradcheck_2d_float64():
                                     eps=1e-6, atol=1e-5, rtol=1e-3, nondet_tol=1e-9)
 
 
+def test_gradcheck_2d_float64_c1_shape():
+    # BASELINE configs[0] at its full shape: N=2, C 8 -> 8, 16x16, k3 p1, one deformable group,
+    # offsets U[-1.5, 1.5] (kept 0.05 away from integer coordinates, where the sampler has kinks).
+    # Full Jacobians (fast_mode off): 13.9k perturbed inputs against 4096 outputs.
+    print("gradcheck 2d c1 shape", flush=True)
+    dcn = _dcn()
+    g = torch.Generator().manual_seed(17)
+    dev = "cuda:0"
+    x = torch.randn(2, 8, 16, 16, generator=g, dtype=torch.float64).to(dev).requires_grad_(True)
+    off = torch.rand(2, 18, 16, 16, generator=g, dtype=torch.float64) * 3 - 1.5
+    off = torch.where((off - off.round()).abs() < 0.05, off + 0.1, off).to(dev).requires_grad_(True)
+    w = (torch.randn(8, 8, 3, 3, generator=g, dtype=torch.float64) * math.sqrt(2.0 / 72)).to(dev).requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda a, b, c: dcn.ConvOffset2dFunction.apply(a, b, c, None, (1, 1), (1, 1), (1, 1), 8, 1),
+                                    (x, off, w), eps=1e-6, atol=1e-5, rtol=1e-3, nondet_tol=1e-9, fast_mode=False)
+
+
 def test_gradcheck_2d_reference_script_shape():
     # deform2d_double/test_gradient.py:7-53
     print("gradcheck 2d ref", flush=True)
@@ -267,6 +283,33 @@ def test_non_finite_and_huge_offsets(name, dtype):
     for nm, g, w in zip(("output", "grad_input", "grad_offset", "grad_weight", "grad_bias"), got, want):
         assert torch.isfinite(g).all(), nm
         assert rel_err(g, w) < TOL[dtype]["fwd" if nm == "output" else "grad"], nm
+
+
+@pytest.mark.parametrize("where", ["grad_output", "weight"])
+@pytest.mark.parametrize("name", ["3d_basic", "2d_basic", "3d_c4_like"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+def test_non_finite_grad_output_and_weight_propagate(name, dtype, where):
+    """NaN / infinite entries of grad_output or of the weight reach the gradients as in the
+    reference's float atomics: where the oracle's gradient is not finite the GPU's is not finite
+    either, and where it is finite the values agree."""
+    print("non-finite", name, dtype, where, flush=True)
+    c = make_case(*SMALL_CASES[name], dtype=dtype, seed=6)
+    t = c["gout"] if where == "grad_output" else c["w"]
+    flat = t.view(-1)
+    idx = torch.randperm(flat.numel(), generator=torch.Generator().manual_seed(2))[:3]
+    flat[idx] = torch.tensor([float("nan"), float("inf"), -float("inf")], dtype=dtype)
+    got = run_gpu(c)
+    want = run_oracle(c)
+    for nm, g, w in zip(("output", "grad_input", "grad_offset", "grad_weight", "grad_bias"), got, want):
+        g = g.detach().cpu().double()
+        w = w.double()
+        fin = torch.isfinite(w)
+        assert torch.equal(torch.isfinite(g), fin), "%s: non-finite mask differs (%d vs %d finite)" % (
+            nm, int(torch.isfinite(g).sum()), int(fin.sum()))
+        if fin.any():
+            scale = w[fin].abs().max().item()
+            tol = TOL[dtype]["fwd" if nm == "output" else "grad"]
+            assert (g[fin] - w[fin]).abs().max().item() <= tol * (scale if scale > 0 else 1.0), nm
 
 
 @pytest.mark.parametrize("name", ["2d_c3_like", "2d_rect_kernel_stride_dil", "3d_dilation3", "3d_basic"])
@@ -450,13 +493,10 @@ def test_needs_input_grad_gating():
 
 
 # ---------------------------------------------------------------------------------------------
-# BASELINE.json sizes.  The oracle is too slow for the whole batch, so: (1) sample 0 of the batch
-# is compared with the oracle run on that sample alone (samples are independent), for a
-# depth-reduced c4 and for c2/c3 at one sample; (2) at full size the bilinear-form identities
-# <out, g> = <x, grad_input> = <W, grad_weight> (for fixed offsets, no bias) are checked.
+# BASELINE.json sizes: the whole batch at full size against the oracle (all four tensors), and the
+# bilinear-form identities <out, g> = <x, grad_input> = <W, grad_weight> (fixed offsets, no bias).
 
 FULL = {
-    # name: (make_case args, oracle batch slice)
     "c2_2d_f32": (2, 8, 256, 256, 56, 3, 1, 1, 1, 256, 1, 2.0),
     "c3_2d_f32_grouped_dilated": (2, 4, 512, 512, 28, 3, 1, 2, 2, 128, 2, None),
     "c4_3d_f32": (3, 4, 64, 64, (16, 56, 56), 3, 1, 1, 1, 64, 1, 1.5),
@@ -464,15 +504,18 @@ FULL = {
 }
 
 
-@pytest.mark.parametrize("name", sorted(FULL))
-def test_full_size_identities_and_sample_parity(name):
-    print("full-size", name, flush=True)
+def full_case(name, seed=0):
     args = FULL[name]
-    kw = dict(dtype=torch.float32, seed=0, bias=False)
+    kw = dict(dtype=torch.float32, seed=seed, bias=False)
     if args[-1] is None:
-        c = make_case(*args[:-1], 1.0, off_dist="normal_mix", **kw)
-    else:
-        c = make_case(*args, **kw)
+        return make_case(*args[:-1], 1.0, off_dist="normal_mix", **kw)
+    return make_case(*args, **kw)
+
+
+@pytest.mark.parametrize("name", sorted(FULL))
+def test_full_size_parity_and_identities(name):
+    print("full-size", name, flush=True)
+    c = full_case(name)
     out, gin, goff, gw, _ = run_gpu(c)
     # identities, accumulated in float64 on the host
     o64, g64 = out.detach().cpu().double(), c["gout"].double()
@@ -482,22 +525,13 @@ def test_full_size_identities_and_sample_parity(name):
     scale = (o64.abs() * g64.abs()).sum().item()
     assert abs(lhs - via_x) / scale < 1e-5, (lhs, via_x, scale)
     assert abs(lhs - via_w) / scale < 1e-5, (lhs, via_w, scale)
-    assert torch.isfinite(goff).all()
-    # one sample against the oracle; 3-D cases are cut to the first output planes to bound CPU time
-    c1 = {k: (v[:1].contiguous() if torch.is_tensor(v) and k in ("x", "off", "gout") else v) for k, v in c.items()}
-    if c["nd"] == 3:
-        # the first sample again on the GPU and the oracle, restricted in depth: both see the same tensors
-        D = 4
-        c1["x"] = c1["x"][:, :, :D].contiguous()
-        c1["off"] = c1["off"][:, :, :D].contiguous()
-        c1["gout"] = c1["gout"][:, :, :D].contiguous()
-        got = run_gpu(c1)
-    else:
-        got = run_gpu(c1)                                    # grad_weight sums over the batch: rerun on the one sample
-    want = run_oracle(c1)
-    for nm, g, w in zip(("output", "grad_input", "grad_offset", "grad_weight"), got, want):
+    # the oracle on the same tensors, whole batch, full extent
+    print("full-size oracle", name, flush=True)
+    want = run_oracle(c)
+    for nm, g, w in zip(("output", "grad_input", "grad_offset", "grad_weight"), (out, gin, goff, gw), want):
         tol = TOL[torch.float32]["fwd" if nm == "output" else "grad"]
         e = rel_err(g, w)
+        print("  %s %s rel err %.2e" % (name, nm, e), flush=True)
         assert e <= tol, "%s %s: relative error %.3e" % (name, nm, e)
 
 
@@ -506,7 +540,7 @@ def test_linearity_in_weight_and_input_full_c4():
     print("linearity c4", flush=True)
     dcn = _dcn()
     dev = "cuda:0"
-    c = make_case(*FULL["c4_3d_f32"], dtype=torch.float32, seed=2, bias=False)
+    c = full_case("c4_3d_f32", seed=2)
     x, off, w1 = c["x"].to(dev), c["off"].to(dev), c["w"].to(dev)
     w2 = torch.randn_like(w1) * w1.std()
     f = lambda xx, ww: dcn.ConvOffset3dFunction.apply(xx, off, ww, None, c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])

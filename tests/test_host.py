@@ -123,8 +123,30 @@ def test_reference_function_script_values():
     assert out[1, 1, 1] == 8.0
     # position (1,0,1): l in {0,2}, h = 1, w in {0,2}: 4 samples of value 2 -> 8
     assert out[1, 0, 1] == 8.0
-    # zero offsets at integer coordinates: grad_offset is the finite difference toward the high corner
     assert d["gw"].shape == (1, 1, 3, 3, 3)
+    # grad_offset by hand.  Weight and grad_output are all ones, so every grad-column value is 1.
+    # A tap at integer coordinate p on an axis: p in {0, 1, 2} is inside; the high corner differs
+    # from the low one only for p = 1 (for p <= 0 and p >= size - 1 it collapses).  The input varies
+    # along h only ([1, 2, 1]), so an inside sample has d/dl = d/dw = 0 and d/dh = x[2] - x[1] = -1
+    # when p_h = 1, else 0.  A sample with any axis outside gets, per axis, -|1| for p <= -1, +|1|
+    # for p >= 3 (the length extent, deform3d/lib/deform_conv3d_cuda_kernel.cu:470-481), else 0.
+    goff = d["goff"].reshape(27, 3, 3, 3, 3)                    # [tap][axis][ol][oh][ow]
+    want = np.zeros_like(goff)
+    for kl in range(3):
+        for kh in range(3):
+            for kw in range(3):
+                tap = (kl * 3 + kh) * 3 + kw
+                for ol in range(3):
+                    for oh in range(3):
+                        for ow in range(3):
+                            p = (ol - 1 + 2 * kl, oh - 1 + 2 * kh, ow - 1 + 2 * kw)
+                            if all(0 <= v <= 2 for v in p):
+                                want[tap, 1, ol, oh, ow] = -1.0 if p[1] == 1 else 0.0
+                            else:
+                                for a in range(3):
+                                    want[tap, a, ol, oh, ow] = -1.0 if p[a] <= -1 else (1.0 if p[a] >= 3 else 0.0)
+    assert np.array_equal(goff, want)
+    assert (want != 0).sum() > 100          # taps at -1 and at 3 (and beyond) do occur
 
 
 def test_pack_modules_construction():
