@@ -193,7 +193,7 @@ static bool fused_chunk8() {      // DCN_FUSED_CHUNK=4: never take 8-channel chu
     return v != 0;
 }
 static int fused_first_waves() {
-    static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : 8; }();
+    static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : (e && atoi(e) == 16) ? 16 : 8; }();
     return v;
 }
 static bool fused_fixed_stride() {      // DCN_FUSED_FIXED=0: runtime plane stride even where the compile-time one fits
@@ -380,8 +380,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
     for (int nw = fused_first_waves(); nw >= 4 && scatter_in_lds() && fused_coord(); nw /= 2) {
         Params Ph = P;
-        if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T), nw, nw != 8)) continue;
-        const size_t tables = (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
+        if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T), nw, nw == 4)) continue;
+        const size_t tables = (size_t)Ph.hvol * 4;      // halo table
         const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
         if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
         if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) < 4) continue;
@@ -435,6 +435,11 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         if constexpr (ND == 2) {
             if (eight) return breg ? DCN_LAUNCH_FUSED_C(8, true, 0, 8) : DCN_LAUNCH_FUSED_C(8, false, 0, 8);
         }
+        if (nw == 16) {      // experimental: 1024 threads, 8x8x8 positions, runtime plane stride
+            if (breg && !eight) { Ph.hstride = (Ph.hvol + 63) / 64 * 64; const size_t lds16 = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + tables;
+                if (lds16 <= 160 * 1024) return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true, 0, 16, true>, "backward_input_halo_kernel", hgrid, 1024, lds16, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit); }
+            continue;
+        }
         if (nw == 8) {
             if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 8);
             if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 8);
@@ -460,7 +465,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
     if (halo && (long long)Ph.N * Ph.tiles * Ph.DG > 0x7fffffffLL) halo = false;
     if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
-        const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4 - (size_t)P.kV * ND * 4) / ((size_t)Ph.hstride * 8);
+        const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * 8);
         if (fit >= 8) Ph.cchunk = 8;
         else if (fit >= 4) Ph.cchunk = 4;
         else halo = false;
@@ -476,7 +481,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             default: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
         }
         if (int rc = check_launch("backward_data_kernel")) return rc;
-        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4 + (size_t)P.kV * ND * 4;
+        const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4;
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG);
         T* nogoff = nullptr;

@@ -9,6 +9,7 @@
 #pragma once
 #include "dcn_device.h"
 
+
 namespace dcn {
 
 constexpr int WG = 256;            // 4 wavefronts
@@ -263,7 +264,7 @@ __device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, 
 
 // The same for a channel-interleaved halo [halo voxel][CCH]: the CCH channel values of a voxel sit
 // next to each other, so one wide LDS read fetches a corner of all of them (missing channels of a
-// short last chunk are stored as zero).
+// short last chunk and halo voxels outside the volume are stored as zero).
 template <typename T, int CCH, int WGS>
 __device__ inline void halo_stage_interleaved(const Params& P, const T* __restrict__ chan0, int nch,
                                               const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
@@ -273,8 +274,9 @@ __device__ inline void halo_stage_interleaved(const Params& P, const T* __restri
         T val[CCH];
 #pragma unroll
         for (int c = 0; c < CCH; ++c) val[c] = chan0[(size_t)min(c, nch - 1) * P.inV + g];   // CCH loads in flight
+        // cells outside the volume hold zero: samples in the rim read them with weight zero
 #pragma unroll
-        for (int c = 0; c < CCH; ++c) sIn[(size_t)v * CCH + c] = c < nch ? val[c] : (T)0;
+        for (int c = 0; c < CCH; ++c) sIn[(size_t)v * CCH + c] = (c < nch && t != ~0u) ? val[c] : (T)0;
     }
 }
 
@@ -883,7 +885,6 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
     T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * hs);                               // [hstride][CCH] if COORD: channels of a voxel side by side
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
-    int* sKd = reinterpret_cast<int*>(sTab + P.hvol);                                   // [kV][ND]: tap * dilation per axis
     constexpr int WGS = NW * 64;                        // threads per workgroup
     __shared__ float sRed[NW];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -906,12 +907,11 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
     halo_table<ND, WGS>(P, tg, sTab);                   // visible after the first barrier below
-    for (int tp = threadIdx.x; tp < P.kV; tp += WGS) {      // taps differ between lanes here: a table replaces the divisions
-        int kk[ND];
-        decode_tap<ND>(P, tp, kk);
+    // o * stride - pad of this lane's position as T: the integer part of a sampling coordinate is
+    // (T)(that + tap * dilation), a sum of two small integers that is exact in T as well
+    T ibf[ND];
 #pragma unroll
-        for (int a = 0; a < ND; ++a) sKd[tp * ND + a] = kk[a] * P.dil[slot<ND>(a)];
-    }
+    for (int a = 0; a < ND; ++a) ibf[a] = (T)ib[a];
 
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
@@ -992,8 +992,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         for (int w8 = 0; w8 < NW; ++w8) smaxb = max(smaxb, __float_as_uint(sRed[w8]));
         int ex = 0;
         const float bound = 8.f * wmax[0] * __uint_as_float(smaxb);
-        // float cells need a finite bound; without one this workgroup scatters through the far path
-        const bool cells_ok = sizeof(T) == 8 || bound < 3.0e38f;      // false for NaN
+        // the LDS cells need a finite bound; without one this workgroup scatters through the far path
+        // (float cells need the exponent; and with either cell type a corner that carries weight zero
+        // would receive 0 * inf = NaN where the reference adds nothing)
+        const bool cells_ok = bound < 3.0e38f;                        // false for NaN
         if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
         const double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
 
@@ -1087,7 +1089,17 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 gemm_tail(d_next, wchunk, 0);
             }
             T o_nx[ND];                                                // offsets and tap * dilation of the next tap slot
-            int kd_nx[ND];
+            T kd_nx[ND];
+            // Kernel coordinates of this lane's tap in the next slot, counted up with the slots (the
+            // taps of consecutive slots are TP / NS apart for every lane).  They live in registers: a
+            // table in LDS would put a read into every slot that can only be waited for together with
+            // the LDS adds issued behind it (LDS operations complete in order and the wait counter
+            // cannot tell conditional adds apart), which serialises the adds with the next slot's
+            // vector work.
+            constexpr int STEP = TP / NS;
+            static_assert(TP % NS == 0, "taps of consecutive slots are evenly spaced");
+            int kq[ND];
+            decode_tap<ND>(P, MM::row(0, q) / CCH, kq);
             auto load_slot_offsets = [&](int tap_u, int ts) {         // tap_u: uniform tap of lane group 0 in slot ts
                 const int tu = min(tap_u, P.kV - 1);
                 const int dq = MM::row(ts * RPS, q) / CCH - MM::row(ts * RPS, 0) / CCH;
@@ -1097,7 +1109,18 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                 for (int a = 0; a < ND; ++a) o_nx[a] = (ob + (size_t)a * P.outV)[lo];
 #pragma unroll
-                for (int a = 0; a < ND; ++a) kd_nx[a] = sKd[(tu + dqc) * ND + a];
+                for (int a = 0; a < ND; ++a) kd_nx[a] = (T)(kq[a] * P.dil[slot<ND>(a)]);
+#pragma unroll
+                for (int st = 0; st < STEP; ++st) {                    // on to the next slot's tap: increment with carry
+                    int carry = 1;
+#pragma unroll
+                    for (int a = ND - 1; a > 0; --a) {
+                        kq[a] += carry;
+                        carry = kq[a] >= P.k[slot<ND>(a)] ? 1 : 0;
+                        kq[a] = carry ? 0 : kq[a];
+                    }
+                    kq[0] += carry;
+                }
             };
             load_slot_offsets(MM::row(0, 0) / CCH, 0);
             // grad_offset of a finished tap slot, held back until the loads of the next slot have been
@@ -1120,6 +1143,13 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 }
                 pend = false;
             };
+            // corner i of a sample sits at a fixed distance from its low corner (strides of the halo);
+            // a corner that the reference collapses onto the low one carries weight zero instead
+            unsigned coff[NC];
+#pragma unroll
+            for (int i = 0; i < NC; ++i)
+                coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * P.hext[1] + ((i >> 1) & 1)) * P.hext[2] + (i & 1))
+                                  : (unsigned)(((i >> 1) & 1) * P.hext[2] + (i & 1));
 
             for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
                 const typename MM::Acc d = d_next;
@@ -1134,10 +1164,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     // slots past the last tap (only in the last pass, which feeds no further MFMAs)
                     if (tap0 + MM::row(ts * RPS, 0) / CCH >= P.kV) continue;
                     const int tap = tap0 + MM::row(ts * RPS, q) / CCH;
-                    T a_cu[AB], b_cu[AB], ofs[ND];
-                    int kd[ND];
+                    T a_cu[AB], b_cu[AB], ofs[ND], kdf[ND];
 #pragma unroll
-                    for (int a = 0; a < ND; ++a) { ofs[a] = o_nx[a]; kd[a] = kd_nx[a]; }
+                    for (int a = 0; a < ND; ++a) { ofs[a] = o_nx[a]; kdf[a] = kd_nx[a]; }
                     const bool do_mma = more && ts * AB < ksteps;      // uniform
                     // this slot's MFMA operands arrive while its geometry is set up; the offsets of the
                     // next tap slot travel while this one is worked on
@@ -1148,132 +1177,184 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     if constexpr (COORD) write_goff();
                     __builtin_amdgcn_sched_barrier(0);
 
-                    TapGeo<T, ND> t;
-                    tap_setup_noidx<T, ND>(P, ofs, ib, kd, t);
+                    // Geometry of this lane's (tap, position), following the reference sampler
+                    // (deform3d/lib/deform_conv3d_cuda_kernel.cu:21-26,40-45,123-124) in a branch-free
+                    // form: the coordinate is clamped into [0, size - 1]; low corner = floor, fraction
+                    // toward the high corner = clamped coordinate - floor.  Where the reference collapses
+                    // the high corner onto the low one (p <= 0, p >= size - 1) the fraction is 0, so the
+                    // corner one step further carries weight 0 (a halo cell outside the volume holds 0)
+                    // and every sample uses the same eight (four) cells at fixed strides.
                     const bool slot_ok = valid && tap < P.kV;
-                    const bool live = slot_ok && t.inside;
+                    bool inside = slot_ok, inhalo = cells_ok;
+                    bool intr[ND];                 // strictly between the collapse zones: the axis has a slope
+                    T pq[ND], f[ND];
+                    int u[ND];                     // low corner in halo coordinates
+#pragma unroll
+                    for (int a = 0; a < ND; ++a) {
+                        const int s = slot<ND>(a);
+                        const T top = (T)(P.in[s] - 1);
+                        const T pa = (ibf[a] + kdf[a]) + ofs[a];
+                        T pc;
+                        if constexpr (sizeof(T) == 4) pc = __builtin_amdgcn_fmed3f(pa, 0.f, top);
+                        else pc = fmin(fmax(pa, (T)0), top);
+                        const T fl = floor(pc);
+                        pq[a] = pa;
+                        f[a] = pc - fl;
+                        inside = inside && fabs(pa - pc) < (T)1;            // -1 < p < size, false for NaN
+                        intr[a] = pa > (T)0 && pa < top;
+                        u[a] = (int)fl - tg.hb[a];
+                        inhalo = inhalo && (unsigned)u[a] < (unsigned)(P.hext[s] - 1);
+                    }
+                    const bool near = inside && inhalo, far = inside && !inhalo;
+                    unsigned base;
+                    if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], P.hext[1]) + u[1], P.hext[2]) + u[2]);
+                    else base = (unsigned)(__mul24(u[0], P.hext[2]) + u[1]);
+                    base = near ? base : 0u;       // lanes without a sample in the halo read cell 0 and add nothing
+                    T cw[NC];
+                    if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
+                        const T fl = f[0], gl = (T)1 - fl, fh = f[1], gh = (T)1 - fh, fw = f[2], gw = (T)1 - fw;
+                        const T a00 = gl * gh, a01 = gl * fh, a10 = fl * gh, a11 = fl * fh;
+                        cw[0] = a00 * gw; cw[1] = a00 * fw; cw[2] = a01 * gw; cw[3] = a01 * fw;
+                        cw[4] = a10 * gw; cw[5] = a10 * fw; cw[6] = a11 * gw; cw[7] = a11 * fw;
+                    } else {
+                        const T fh = f[0], gh = (T)1 - fh, fw = f[1], gw = (T)1 - fw;
+                        cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                    }
+                    // grad-column values of this slot (rows past the chunk's channels: packed weights are
+                    // zero there; the plain layout holds a neighbour's weights, so those are masked)
+                    T gv[RPS];
+#pragma unroll
+                    for (int rr = 0; rr < RPS; ++rr) {
+                        gv[rr] = d[ts * RPS + rr];
+                        if constexpr (!PACKW) gv[rr] = (MM::row(ts * RPS + rr, q) % CCH) < nch ? gv[rr] : (T)0;
+                    }
+                    // corner values of the input: one wide LDS read per corner for all of this lane's
+                    // channels, issued by every lane, ahead of the MFMAs that cover their latency
+                    T vv[NC][RPS];
+                    if constexpr (COORD) {
+                        const T* ip = sIn + (size_t)base * CCH;
+#pragma unroll
+                        for (int i = 0; i < NC; ++i)
+#pragma unroll
+                            for (int rr = 0; rr < RPS; ++rr) vv[i][rr] = ip[coff[i] * CCH + MM::row(ts * RPS + rr, q) % CCH];
+                    }
+                    // the next pass's MFMAs of this slot, in uniform control flow
+                    if (do_mma) {
+#pragma unroll
+                        for (int k = 0; k < AB; ++k)
+                            d_next = MM::mma(a_cu[k], BREG ? b_reg[ts * AB + k] : b_cu[k], d_next);
+                    }
                     T ga[ND];
 #pragma unroll
                     for (int a = 0; a < ND; ++a) ga[a] = 0;
-                    // corner cells and weights, computed by every lane (dead lanes never use them)
-                    unsigned lidx[NC];
-                    const bool in_halo = halo_corners_strided<T, ND>(P, tg.hb, t, lidx) && cells_ok;
-                    T cw[NC];
-                    if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
-                        const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
-                        cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
-                        cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
-                    } else {
-                        const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                        cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
-                    }
-                    double cwd[NC];                // widened once per tap slot, used for every channel
+                    if constexpr (COORD) {
+                        // d(sample)/d(coordinate) is linear in the corner values: it is applied once to
+                        // the corner values weighted by gcol and summed over the lane's channels.  Every
+                        // lane does this, outside any branch (a lane without a near sample works on cell
+                        // 0 and drops the result): corner reads still pending at a branch that skips
+                        // their use would make the compiler wait for the whole LDS queue, adds included,
+                        // before the registers are written again.
+                        T v[NC];
 #pragma unroll
-                    for (int i = 0; i < NC; ++i) cwd[i] = (double)cw[i];
-                    // out-of-range samples of the 3-D operator: +-|gcol| per axis; h and w are compared
-                    // with the LENGTH extent
-                    const bool oor = COORD && ND == 3 && slot_ok && !t.inside && !P.oob_zero;
-                    T sg[ND];
+                        for (int i = 0; i < NC; ++i) {
+                            T acc_ = gv[0] * vv[i][0];
 #pragma unroll
-                    for (int a = 0; a < ND; ++a) sg[a] = (t.p[a] <= (T)-1) ? (T)-1 : ((t.p[a] >= (T)P.in[0]) ? (T)1 : (T)0);
-                    const bool near = live && in_halo, far = live && !in_halo;
-                    // corner cells of channel 0; the other channels are an immediate offset away when the
-                    // plane stride is a compile-time constant
-                    Cell* g_cell[NC];
-                    const T* in_cell[NC];
-#pragma unroll
-                    for (int i = 0; i < NC; ++i) { g_cell[i] = sG + lidx[i]; in_cell[i] = sIn + (size_t)lidx[i] * CCH; }
-                    // d(sample)/d(coordinate) from corner values; the formula is linear in them, so it is
-                    // applied once per tap slot to the corner values weighted by gcol and summed over the
-                    // lane's channels (the w-lerps of the four (l, h) corner pairs are shared by the l
-                    // and h derivatives)
-                    auto coord_grad = [&](const T v[NC]) {
+                            for (int rr = 1; rr < RPS; ++rr) acc_ += gv[rr] * vv[i][rr];
+                            v[i] = acc_;
+                        }
                         if constexpr (ND == 3) {
-                            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                            const T fl = f[0], gl = (T)1 - fl, fh = f[1], gh = (T)1 - fh, fw = f[2], gw = (T)1 - fw;
                             const T c00 = v[0] * gw + v[1] * fw, c01 = v[2] * gw + v[3] * fw;
                             const T c10 = v[4] * gw + v[5] * fw, c11 = v[6] * gw + v[7] * fw;
-                            ga[0] += (c10 - c00) * gh + (c11 - c01) * fh;
-                            ga[1] += (c01 - c00) * gl + (c11 - c10) * fl;
-                            ga[2] += ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
-                                     ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
+                            const T dl = (c10 - c00) * gh + (c11 - c01) * fh;
+                            const T dh = (c01 - c00) * gl + (c11 - c10) * fl;
+                            const T dw = ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                         ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
+                            ga[0] = (near && intr[0]) ? dl : (T)0; ga[1] = (near && intr[1]) ? dh : (T)0;
+                            ga[2] = (near && intr[2]) ? dw : (T)0;
                         } else {
-                            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
-                            ga[0] += (v[2] - v[0]) * gw + (v[3] - v[1]) * fw;
-                            ga[1] += (v[1] - v[0]) * gh + (v[3] - v[2]) * fh;
+                            const T fh = f[0], gh = (T)1 - fh, fw = f[1], gw = (T)1 - fw;
+                            const T dh = (v[2] - v[0]) * gw + (v[3] - v[1]) * fw;
+                            const T dw = (v[1] - v[0]) * gh + (v[3] - v[2]) * fh;
+                            ga[0] = (near && intr[0]) ? dh : (T)0; ga[1] = (near && intr[1]) ? dw : (T)0;
                         }
-                    };
-                    // corner values of the input, one wide LDS read per corner for all of this lane's
-                    // channels, weighted by their grad-column values.  The reads go first: LDS operations
-                    // complete in order, so this waits for them only, not for the adds issued below
-                    T gsum[NC];
-                    if constexpr (COORD) {
-                        if (near) {
-                            T gvc[RPS];
+                    }
+                    if (near) {
+                        Cell* cp = sG + base;
 #pragma unroll
-                            for (int rr = 0; rr < RPS; ++rr)
-                                gvc[rr] = (MM::row(ts * RPS + rr, q) % CCH) < nch ? d[ts * RPS + rr] : (T)0;
-                            // every corner's read is issued before the first is used: one wait for
-                            // the LDS queue (the previous slot's adds are ahead in it) instead of one
-                            // per pair of reads
-                            T vv[NC][RPS];
+                        for (int rr = 0; rr < RPS; ++rr) {
+                            const double gs = LdsCell<T>::pre(gv[rr], scale);
+                            const int cl = MM::row(ts * RPS + rr, q) % CCH;
 #pragma unroll
-                            for (int i = 0; i < NC; ++i)
+                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(cp + coff[i] + cl * hs, (double)cw[i], gs);
+                        }
+                    }
+                    if constexpr (COORD && ND == 3) {
+                        // out-of-range samples of the 3-D operator: -|gcol| per axis with p <= -1, +|gcol|
+                        // with p >= the LENGTH extent (h and w are compared with it too), summed over the
+                        // channels (deform3d/lib/deform_conv3d_cuda_kernel.cu:470-481).  Selected, not
+                        // multiplied: 0 * inf would be NaN where the reference adds nothing
+                        const bool oor = slot_ok && !inside && !P.oob_zero;
+                        if (__any(oor)) {
+                            T asum = 0;
 #pragma unroll
-                                for (int rr = 0; rr < RPS; ++rr) vv[i][rr] = in_cell[i][MM::row(ts * RPS + rr, q) % CCH];
-                            __builtin_amdgcn_sched_barrier(0);
+                            for (int rr = 0; rr < RPS; ++rr) asum += fabs(gv[rr]);
+                            if (oor) {
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) {
-                                T acc_ = 0;
-#pragma unroll
-                                for (int rr = 0; rr < RPS; ++rr) acc_ += gvc[rr] * vv[i][rr];
-                                gsum[i] = acc_;
+                                for (int a = 0; a < ND; ++a)
+                                    ga[a] = pq[a] <= (T)-1 ? -asum : (pq[a] >= (T)P.in[0] ? asum : (T)0);
                             }
                         }
                     }
-#pragma unroll
-                    for (int rr = 0; rr < RPS; ++rr) {
-                        const int r = ts * RPS + rr;
-                        const int cl = MM::row(r, q) % CCH;
-                        const T gv = d[r];
-                        if (cl >= nch) {
-                        } else if (near) {
-                            const double gs = LdsCell<T>::pre(gv, scale);
-#pragma unroll
-                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(g_cell[i] + cl * hs, cwd[i], gs);
-                        } else if (oor) {
-                            const T av = gv > 0 ? gv : -gv;
-#pragma unroll
-                            for (int a = 0; a < ND; ++a)      // selected, not multiplied: 0 * inf would be NaN where the reference adds nothing
-                                ga[a] += sg[a] < (T)0 ? -av : (sg[a] > (T)0 ? av : (T)0);
-                        }
-                        // the next pass's MFMAs of this step, in uniform control flow
-                        if (do_mma) {
-#pragma unroll
-                            for (int k = 0; k < MPR; ++k)
-                                d_next = MM::mma(a_cu[rr * MPR + k], BREG ? b_reg[ts * AB + rr * MPR + k] : b_cu[rr * MPR + k], d_next);
-                        }
-                    }
-                    if constexpr (COORD) {
-                        if (near) coord_grad(gsum);
-                    }
                     if (__any(far)) {              // rare: samples that reach past the halo go to global memory
+                        TapGeo<T, ND> t;           // the reference's corner rule on the same coordinate
+                        t.inside = far;
+#pragma unroll
+                        for (int a = 0; a < ND; ++a) {
+                            const T pa = pq[a];
+                            const int l = far ? (int)pa : 0;
+                            t.p[a] = pa;
+                            t.lo[a] = l;
+                            t.hi[a] = (pa >= (T)(P.in[slot<ND>(a)] - 1) || pa <= (T)0) ? l : l + 1;
+                            t.f[a] = pa - (T)l;
+                        }
                         tap_corner_idx<T, ND>(P, t);
+                        T fcw[NC];
+                        if constexpr (ND == 3) {
+                            const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                            fcw[0] = gl * gh * gw; fcw[1] = gl * gh * fw; fcw[2] = gl * fh * gw; fcw[3] = gl * fh * fw;
+                            fcw[4] = fl * gh * gw; fcw[5] = fl * gh * fw; fcw[6] = fl * fh * gw; fcw[7] = fl * fh * fw;
+                        } else {
+                            const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                            fcw[0] = gh * gw; fcw[1] = gh * fw; fcw[2] = fh * gw; fcw[3] = fh * fw;
+                        }
 #pragma unroll
                         for (int rr = 0; rr < RPS; ++rr) {
-                            const int r = ts * RPS + rr;
-                            const int cl = MM::row(r, q) % CCH;
+                            const int cl = MM::row(ts * RPS + rr, q) % CCH;
                             if (far && cl < nch) {
-                                const T gv = d[r];
+                                const T g1 = gv[rr];
                                 const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
                                 T* gc = gin + chan;
 #pragma unroll
-                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], (T)cwd[i] * gv);
+                                for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], fcw[i] * g1);
                                 if constexpr (COORD) {
                                     const T* ic = in + chan;
                                     T v[NC];
 #pragma unroll
-                                    for (int i = 0; i < NC; ++i) v[i] = gv * ic[t.idx[i]];
-                                    coord_grad(v);
+                                    for (int i = 0; i < NC; ++i) v[i] = g1 * ic[t.idx[i]];
+                                    if constexpr (ND == 3) {
+                                        const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                                        const T c00 = v[0] * gw + v[1] * fw, c01 = v[2] * gw + v[3] * fw;
+                                        const T c10 = v[4] * gw + v[5] * fw, c11 = v[6] * gw + v[7] * fw;
+                                        ga[0] += (c10 - c00) * gh + (c11 - c01) * fh;
+                                        ga[1] += (c01 - c00) * gl + (c11 - c10) * fl;
+                                        ga[2] += ((v[1] - v[0]) * gh + (v[3] - v[2]) * fh) * gl +
+                                                 ((v[5] - v[4]) * gh + (v[7] - v[6]) * fh) * fl;
+                                    } else {
+                                        const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                                        ga[0] += (v[2] - v[0]) * gw + (v[3] - v[1]) * fw;
+                                        ga[1] += (v[1] - v[0]) * gh + (v[3] - v[2]) * fh;
+                                    }
                                 }
                             }
                         }
