@@ -1088,8 +1088,11 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             } else {
                 gemm_tail(d_next, wchunk, 0);
             }
-            T o_nx[ND];                                                // offsets and tap * dilation of the next tap slot
-            T kd_nx[ND];
+            // offsets and tap * dilation of the current and of the next tap slot, in two register sets
+            // that swap roles from slot to slot (NS is even): copying "next" into "current" would have
+            // to wait for the loads at the copy, a whole slot before the values are needed
+            T o_buf[2][ND], kd_buf[2][ND];
+            static_assert(NS % 2 == 0, "offset buffers alternate within a pass");
             // Kernel coordinates of this lane's tap in the next slot, counted up with the slots (the
             // taps of consecutive slots are TP / NS apart for every lane).  They live in registers: a
             // table in LDS would put a read into every slot that can only be waited for together with
@@ -1101,6 +1104,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             int kq[ND];
             decode_tap<ND>(P, MM::row(0, q) / CCH, kq);
             auto load_slot_offsets = [&](int tap_u, int ts) {         // tap_u: uniform tap of lane group 0 in slot ts
+                T* o_nx = o_buf[ts & 1];
+                T* kd_nx = kd_buf[ts & 1];
                 const int tu = min(tap_u, P.kV - 1);
                 const int dq = MM::row(ts * RPS, q) / CCH - MM::row(ts * RPS, 0) / CCH;
                 const int dqc = tu + dq < P.kV ? dq : 0;
@@ -1164,9 +1169,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     // slots past the last tap (only in the last pass, which feeds no further MFMAs)
                     if (tap0 + MM::row(ts * RPS, 0) / CCH >= P.kV) continue;
                     const int tap = tap0 + MM::row(ts * RPS, q) / CCH;
-                    T a_cu[AB], b_cu[AB], ofs[ND], kdf[ND];
-#pragma unroll
-                    for (int a = 0; a < ND; ++a) { ofs[a] = o_nx[a]; kdf[a] = kd_nx[a]; }
+                    T a_cu[AB], b_cu[AB];
+                    const T* ofs = o_buf[ts & 1];
+                    const T* kdf = kd_buf[ts & 1];
                     const bool do_mma = more && ts * AB < ksteps;      // uniform
                     // this slot's MFMA operands arrive while its geometry is set up; the offsets of the
                     // next tap slot travel while this one is worked on
