@@ -36,6 +36,8 @@ def load():
     L.dcn_last_error.restype = ctypes.c_char_p
     L.dcn_workspace_bytes.restype = _c_sz
     L.dcn_workspace_bytes.argtypes = [_c_int] * 4 + [_c_sz, _c_sz, _c_int, _c_int]
+    L.dcn_workspace_bytes_for.restype = _c_sz
+    L.dcn_workspace_bytes_for.argtypes = [_c_int] * 4 + [_c_sz, _c_sz, _c_int, _c_int, _c_int]
     tail = [_c_vp, _c_sz, _c_vp]            # workspace, workspace_bytes, stream
     for nd in (2, 3):
         geom = [_c_int] * N_GEOM[nd]
@@ -60,7 +62,7 @@ def check(rc):
         raise DcnError(load().dcn_last_error().decode())
 
 
-EXPORTS = ["dcn_version", "dcn_arch", "dcn_last_error", "dcn_workspace_bytes"] + [
+EXPORTS = ["dcn_version", "dcn_arch", "dcn_last_error", "dcn_workspace_bytes", "dcn_workspace_bytes_for"] + [
     "dcn%dd_%s_%s" % (nd, op, suf)
     for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight") for suf in ("f32", "f64")] + [
     "dcn3d_backward_input_offset_flags_f32", "dcn3d_backward_input_offset_flags_f64"]

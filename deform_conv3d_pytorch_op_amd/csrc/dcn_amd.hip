@@ -3,6 +3,7 @@
 // work is enqueued on the caller's stream.
 #include "../../include/dcn_amd.h"
 #include "dcn_kernels.h"
+#include "dcn_forward.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -56,25 +57,33 @@ template <typename T> size_t packed_weight_elems(int M, int kV, size_t slabs, in
     const int KL = Mma<T>::KL, TP = Mma<T>::TN / cch;
     return slabs * ((kV + TP - 1) / TP) * (size_t)(((M + KL - 1) / KL + 7) / 8 * 8) * 64;
 }
-// Either weight layout of backward_input_offset fits.  The slab count of the packed one depends on
-// the deformable groups, which the workspace query is not told: it is bounded by their largest
-// possible number, C_in.
-template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G) {
+// Upper bound of chunk_slot<cch>(cpg, Cg, c) + 1 over the channels: the slabs a per-chunk weight
+// layout occupies.  cpg = 0: the channels per deformable group are not known (the first workspace
+// query is not told them) and the bound assumes their largest possible number of groups, C_in.
+size_t slab_bound(size_t C_in, int G, int cpg, int cch) { return C_in / cch + (cpg > 0 ? C_in / cpg : C_in) + G + 1; }
+// Either weight layout of backward_input_offset fits.
+template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G, int cpg = 0) {
     int Mp, Cgp;
     bwd_data_weight_pad<T>(M, Cg, Mp, Cgp);
     const size_t plain = ((size_t)G * kV + TAP_PAD) * Mp * Cgp;
     const size_t C_in = (size_t)Cg * G;
-    const size_t packed4 = packed_weight_elems<T>(M, kV, C_in / 4 + C_in + G + 1, 4);
-    const size_t packed8 = packed_weight_elems<T>(M, kV, C_in / 8 + C_in + G + 1, 8);
+    const size_t packed4 = packed_weight_elems<T>(M, kV, slab_bound(C_in, G, cpg, 4), 4);
+    const size_t packed8 = packed_weight_elems<T>(M, kV, slab_bound(C_in, G, cpg, 8), 8);
     const size_t packed = packed4 > packed8 ? packed4 : packed8;
     return align256((plain > packed ? plain : packed) * sizeof(T));
 }
-template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G) {
+template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G, int cpg = 0) {
     const int M = C_out / G, Cg = C_in / G;
     int MT, mchunks, Mp, Cgp;
     fwd_weight_pad<T>(M, Cg, MT, mchunks, Mp, Cgp);
-    const size_t fwd = (size_t)G * kV * Mp * Cgp * sizeof(T);
-    const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
+    // forward: [g][tap][c][m] for the kernel without LDS tiling, or one slab per four channels for the
+    // halo kernel (its row padding is at most eight tiles' worth)
+    const int TNf = Mma<T>::TN;
+    const int Mp8 = ((M + TNf - 1) / TNf + 7) / 8 * 8 * TNf;
+    const size_t fwd_plain = (size_t)G * kV * (Mp > Mp8 ? Mp : Mp8) * Cgp * sizeof(T);
+    const size_t fwd_quad = slab_bound((size_t)C_in, G, cpg, FQ) * forward_slab_elems<T>(kV, Mp8) * sizeof(T);
+    const size_t fwd = fwd_plain > fwd_quad ? fwd_plain : fwd_quad;
+    const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G, cpg) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
     // backward_weight: two channels-last copies + one partial weight per position split (at most 256 splits,
     // and never more than about 4096 workgroups: see bww_plan)
     const int TNq = Mma<T>::TN;
@@ -218,7 +227,7 @@ int halo_margin() {
 
 template <typename T, int ND>
 bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH,
-               bool smallest_halo = false) {
+               bool smallest_halo = false, int chunk_mult = 0) {
     const int npos = waves * Mma<T>::TN;        // positions per workgroup, one column tile per wavefront
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
@@ -252,7 +261,7 @@ bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_by
     if (hvol > MAX_HVOL) return false;
     P.hvol = (int)hvol;
     P.hstride = ((int)hvol + 63) / 64 * 64 + 32;
-    const int KL = Mma<T>::KL;
+    const int KL = chunk_mult > 0 ? chunk_mult : Mma<T>::KL;      // channels per pass come in multiples of this
     if (budget <= (size_t)hvol * 4) return false;
     long long cc = (long long)((budget - (size_t)hvol * 4) / ((size_t)P.hstride * cell_bytes));
     cc = cc / KL * KL;
@@ -304,33 +313,53 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
         }
         P.Mp = P.mchunks * MT * TN;
     }
+    // Halo kernel: four channels of a voxel side by side in LDS (forward_quad_kernel).  Few
+    // accumulators (MT <= 2): one 1024-thread workgroup per CU with the whole LDS, if its larger halo
+    // fits and leaves 8 channels per pass.  Otherwise 512 threads: two workgroups per CU when that
+    // still leaves 8 channels per LDS pass, else one large one.
+    {
+        Params Ph = P;
+        int nw = 0;
+        // (the 3-D double instance of the 1024-thread shape does not fit its 128 registers)
+        if (MT <= 2 && wide_forward() && !(sizeof(T) == 8 && ND == 3)) {
+            Params Pw = P;
+            if (plan_halo<T, ND>(Pw, 144 * 1024, 1 << 30, sizeof(T), 16, false, FQ) &&
+                (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks <= 0x7fffffffLL &&
+                (wide_forward() == 2 || (Pw.cchunk >= 8 && (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks >= cu_count()))) {
+                Ph = Pw;
+                nw = 16;
+            }
+        }
+        if (!nw) {
+            bool tiled = plan_halo<T, ND>(Ph, LDS_BUDGET, 1 << 30, sizeof(T), WAVESH, false, FQ);
+            if ((!tiled || Ph.cchunk < 8) && LDS_BUDGET < 144 * 1024)
+                tiled = plan_halo<T, ND>(Ph, 144 * 1024, 1 << 30, sizeof(T), WAVESH, false, FQ) || tiled;
+            if (tiled && (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks <= 0x7fffffffLL) nw = WAVESH;
+        }
+        const size_t slabs = (size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1;
+        const size_t wq_bytes = slabs * forward_slab_elems<T>(P.kV, P.Mp) * sizeof(T);
+        if (nw && ws_bytes >= wq_bytes) {
+            {
+                const size_t total = (size_t)P.C_in * forward_slab_elems<T>(P.kV, P.Mp);
+                const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
+                hipLaunchKernelGGL(pack_forward_weight_kernel<T>, dim3(blocks), dim3(256), 0, s, Ph, w, wt);
+                if (int rc = check_launch("pack_forward_weight_kernel")) return rc;
+            }
+            const size_t lds = (size_t)Ph.cchunk * Ph.hstride * sizeof(T) + (size_t)Ph.hvol * 4;
+            const dim3 grid((unsigned)Ph.N * Ph.tiles * Ph.G * Ph.mchunks);
+            if (nw == 16) {
+                if (MT == 1) return launch_halo(forward_quad_kernel<T, ND, 1, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, bias, out);
+                return launch_halo(forward_quad_kernel<T, ND, 2, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, bias, out);
+            }
+            switch (MT) {
+                case 1: return launch_halo(forward_quad_kernel<T, ND, 1, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
+                case 2: return launch_halo(forward_quad_kernel<T, ND, 2, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
+                case 4: return launch_halo(forward_quad_kernel<T, ND, 4, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
+                default: return launch_halo(forward_quad_kernel<T, ND, 8, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
+            }
+        }
+    }
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
-    // Few accumulators (MT <= 2): one 1024-thread workgroup per CU with the whole LDS, if its larger
-    // halo fits and leaves 8 channels per pass.  Otherwise 512 threads: two workgroups per CU when
-    // that still leaves 8 channels per LDS pass, else one large one.
-    if (MT <= 2 && wide_forward()) {
-        Params Pw = P;
-        if (plan_halo<T, ND>(Pw, 144 * 1024, 1 << 30, sizeof(T), 16) &&
-            (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks <= 0x7fffffffLL &&
-            (wide_forward() == 2 || (Pw.cchunk >= 8 && (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks >= cu_count()))) {
-            const size_t lds = (size_t)Pw.cchunk * Pw.hstride * sizeof(T) + (size_t)Pw.hvol * 4;
-            const dim3 grid((unsigned)Pw.N * Pw.tiles * Pw.G * Pw.mchunks);
-            if (MT == 1) return launch_halo(forward_halo_kernel<T, ND, 1, 16>, "forward_halo_kernel", grid, 1024, lds, s, Pw, in, off, wt, bias, out);
-            return launch_halo(forward_halo_kernel<T, ND, 2, 16>, "forward_halo_kernel", grid, 1024, lds, s, Pw, in, off, wt, bias, out);
-        }
-    }
-    bool tiled = plan_halo<T, ND>(P, LDS_BUDGET);
-    if ((!tiled || P.cchunk < 8) && LDS_BUDGET < 144 * 1024) tiled = plan_halo<T, ND>(P, 144 * 1024) || tiled;
-    if (tiled && (long long)P.N * P.tiles * P.G * P.mchunks <= 0x7fffffffLL) {
-        const size_t lds = (size_t)P.cchunk * P.hstride * sizeof(T) + (size_t)P.hvol * 4;
-        const dim3 grid((unsigned)P.N * P.tiles * P.G * P.mchunks);
-        switch (MT) {
-            case 1: return launch_halo(forward_halo_kernel<T, ND, 1, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
-            case 2: return launch_halo(forward_halo_kernel<T, ND, 2, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
-            case 4: return launch_halo(forward_halo_kernel<T, ND, 4, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
-            default: return launch_halo(forward_halo_kernel<T, ND, 8, WAVESH>, "forward_halo_kernel", grid, WGH, lds, s, P, in, off, wt, bias, out);
-        }
-    }
     // geometry whose halo does not fit in LDS: gather straight from global memory
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
@@ -361,7 +390,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     P.oob_zero = (flags & DCN_FLAG_OOB_OFFSET_GRAD_ZERO) ? 1 : 0;
     if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     bwd_data_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
-    const size_t wbytes = bwd_data_weight_bytes<T>(P.M, P.Cg, P.kV, P.G);
+    const size_t wbytes = bwd_data_weight_bytes<T>(P.M, P.Cg, P.kV, P.G, P.cpg);
     const size_t tbytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
     if (!ws || ws_bytes < wbytes + 2 * tbytes) return fail(DCN_E_WORKSPACE, "workspace too small");
     T* wt = static_cast<T*>(ws);
@@ -655,6 +684,17 @@ size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, 
     return elem_size == 8
                ? workspace_need<double>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group)
                : workspace_need<float>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group);
+}
+
+size_t dcn_workspace_bytes_for(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
+                               size_t output_volume, int kernel_volume, int group, int channel_per_deformable_group) {
+    if (group <= 0 || batch <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0 || input_volume == 0 ||
+        output_volume == 0 || channel_per_deformable_group <= 0 || input_c % channel_per_deformable_group)
+        return 0;
+    const int cpg = channel_per_deformable_group;
+    return elem_size == 8
+               ? workspace_need<double>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg)
+               : workspace_need<float>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg);
 }
 
 #define DEFINE_OPS(SUF, T)                                                                                          \

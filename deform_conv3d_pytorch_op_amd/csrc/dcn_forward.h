@@ -1,0 +1,303 @@
+// Forward kernel with the input halo in LDS, four channels of a voxel side by side.
+//
+//   out[n][g*M + m][pos] = sum_{cl,tap} W[g*M+m][cl][tap] * sample(in[n][g*Cg+cl], tap, pos)  (+ bias)
+//
+// replaces deformable_im2col + the per-group Sgemm of the reference
+// (deform3d/lib/deform_conv3d_cuda.cpp:110-148, deform2d_double/lib/deform_conv2d_cuda.cpp:102-138).
+//
+// Lane roles.  A wavefront owns TN output positions; lane (j, q) works on position j and on
+// reduction slot q of the MFMA (B[k = q][col = j]).  The KL reduction slots of one MFMA step are KL
+// consecutive TAPS of one channel: lane group q samples tap tg*KL + q, so every lane derives the
+// geometry of ONE (tap, position) per tap group and no two lanes of a wavefront repeat each other's
+// work.  The sample then serves four channels at a time: the halo holds the four channels of a
+// voxel in 16 (32) consecutive bytes, one wide LDS read per corner fetches all of them, and the
+// interpolated values of the four channels are the B operands of four MFMA steps.
+#pragma once
+#include "dcn_kernels.h"
+
+namespace dcn {
+
+constexpr int FQ = 4;              // channels per group: one wide LDS read per corner
+
+// Weights of the forward kernel: one slab per group of four channels (groups start at the first
+// channel of a segment -- the channels shared by one deformable group and one convolution group --
+// and every fourth after it), in the order the lanes consume them:
+//   Wq[slab][tap group][row tile][q][j][e] = W[m = tile*TN + j][channel = first + e][tap = tg*KL + q]
+// zero past M, past the last tap and past the segment.  A lane's four values of one (tap group, row
+// tile) are 16 (32) contiguous bytes and a wavefront's are one contiguous run.
+template <typename T>
+__host__ __device__ inline size_t forward_slab_elems(int kV, int Mp) {
+    return (size_t)((kV + Mma<T>::KL - 1) / Mma<T>::KL) * Mp * Mma<T>::KL * FQ;
+}
+
+template <typename T>
+__global__ void pack_forward_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wq) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL;
+    const int mtiles = P.Mp / TN;
+    const size_t per_slab = forward_slab_elems<T>(P.kV, P.Mp);
+    const size_t total = (size_t)P.C_in * per_slab;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int c0 = (int)(i / per_slab);                    // candidate first channel of a group
+        const int seg_b = max(c0 / P.cpg * P.cpg, c0 / P.Cg * P.Cg);
+        if ((c0 - seg_b) % FQ) continue;
+        const int seg_e = min((c0 / P.cpg + 1) * P.cpg, (c0 / P.Cg + 1) * P.Cg);
+        size_t r = i % per_slab;
+        const int e = (int)(r % FQ); r /= FQ;
+        const int j = (int)(r % TN); r /= TN;
+        const int q = (int)(r % KL); r /= KL;
+        const int tile = (int)(r % mtiles);
+        const int tg = (int)(r / mtiles);
+        const int m = tile * TN + j, tap = tg * KL + q, c = c0 + e, g = c0 / P.Cg;
+        T v = 0;
+        if (m < P.M && tap < P.kV && c < seg_e) v = W[(((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap];
+        Wq[(size_t)chunk_slot<FQ>(P.cpg, P.Cg, c0) * per_slab + i % per_slab] = v;
+    }
+}
+
+// Stage `nch` channels of the halo as groups of four: sIn[group][halo voxel][4].  Missing channels
+// of a short last group and halo voxels outside the volume hold zero (a sample in the rim reads
+// the latter with weight zero).
+template <typename T, int WGS>
+__device__ inline void halo_stage_quads(const Params& P, const T* __restrict__ chan0, int nch,
+                                        const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
+    const int ngrp = (nch + FQ - 1) / FQ;
+    for (int v = threadIdx.x; v < P.hvol; v += WGS) {
+        const unsigned t = sTab[v];
+        const unsigned g = t == ~0u ? 0u : t;
+        for (int grp = 0; grp < ngrp; ++grp) {
+            T val[FQ];
+#pragma unroll
+            for (int e = 0; e < FQ; ++e) val[e] = chan0[(size_t)min(grp * FQ + e, nch - 1) * P.inV + g];
+#pragma unroll
+            for (int e = 0; e < FQ; ++e)
+                sIn[((size_t)grp * P.hstride + v) * FQ + e] = (grp * FQ + e < nch && t != ~0u) ? val[e] : (T)0;
+        }
+    }
+}
+
+// 1-D grid of N * tiles (3-D blocks of positions) * G * mchunks workgroups of NW wavefronts;
+// dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4 with cchunk a multiple of four.
+template <typename T, int ND, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void forward_quad_kernel(Params P, const T* __restrict__ in,
+                                                           const T* __restrict__ off, const T* __restrict__ Wq,
+                                                           const T* __restrict__ bias, T* __restrict__ out) {
+    using MM = Mma<T>;
+    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, WGS = NW * 64;
+    typedef T V4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sIn = reinterpret_cast<T*>(smem_raw);                                            // [cchunk / 4][hstride][4]
+    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)P.cchunk * P.hstride);   // [hvol]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % TN, q = lane / TN;
+    // workgroups of one tile are neighbours in an XCD-contiguous order
+    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+    const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
+    const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
+
+    TileGeo<ND> tg_;
+    tile_decode<ND>(P, wg / (unsigned)(P.G * P.mchunks), tg_);
+    const int n = tg_.n;
+    int o[ND];
+    unsigned pos;
+    const bool valid = tile_position<ND>(P, tg_, wave * TN + j, o, pos);
+    // o * stride - pad as T: the integer part of a sampling coordinate is (T)(that + tap * dilation),
+    // a sum of two small integers that is exact in T as well
+    T ibf[ND];
+#pragma unroll
+    for (int a = 0; a < ND; ++a) ibf[a] = (T)(o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)]);
+    halo_table<ND, WGS>(P, tg_, sTab);             // visible after the first barrier below
+
+    typename MM::Acc acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
+
+    const int ntg = (P.kV + KL - 1) / KL, mtiles = P.Mp / TN;
+    const size_t per_slab = forward_slab_elems<T>(P.kV, P.Mp);
+    // corner i of a sample sits at a fixed distance from its low corner (strides of the halo); a
+    // corner that the reference collapses onto the low one carries weight zero instead
+    unsigned coff[NC];
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+        coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * P.hext[1] + ((i >> 1) & 1)) * P.hext[2] + (i & 1))
+                          : (unsigned)(((i >> 1) & 1) * P.hext[2] + (i & 1));
+    // this lane's weights of (tap group 0, first row tile of the chunk) inside a slab
+    const unsigned w_lane = (((unsigned)mchunk * MT * KL + q) * TN + j) * FQ;
+    const unsigned w_tile = (unsigned)KL * TN * FQ;               // one row tile further
+    const unsigned w_tg = (unsigned)mtiles * KL * TN * FQ;        // one tap group further
+
+    const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
+    for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+        const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
+        const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+        for (int cc0 = cb; cc0 < ce; cc0 += P.cchunk) {
+            const int nch = min(P.cchunk, ce - cc0);
+            const int ngrp = (nch + FQ - 1) / FQ;
+            const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
+            __syncthreads();                                               // readers of the previous chunk are done
+            halo_stage_quads<T, WGS>(P, chan0, nch, sTab, sIn);
+            __syncthreads();
+            // slabs of consecutive groups of one segment are consecutive.  Uniform base (scalar
+            // registers); the lanes add the 32-bit offset w_lane.
+            const T* wchunk = Wq + (size_t)chunk_slot<FQ>(P.cpg, P.Cg, cc0) * per_slab;
+
+            // kernel coordinates of this lane's tap, counted up with the tap groups
+            int kq[ND];
+            decode_tap<ND>(P, q, kq);
+            T o_buf[2][ND];
+            auto load_offsets_of = [&](int tgi, T* dst) {                  // offsets of tap tgi*KL + q (clamped to a legal tap)
+                const T* ob = off_dg + (size_t)tgi * KL * ND * P.outV;     // uniform
+                const unsigned lo = (unsigned)min(q, P.kV - 1 - tgi * KL) * ND * P.outV + pos;
+#pragma unroll
+                for (int a = 0; a < ND; ++a) dst[a] = (ob + (size_t)a * P.outV)[lo];
+            };
+            load_offsets_of(0, o_buf[0]);
+
+            // One tap group: geometry of this lane's (tap, position), then per group of four channels
+            // eight (four) wide corner reads, the weighted corner sums and 4 * MT MFMAs.
+            auto tap_group = [&](int tgi, const T* ofs) {
+                const bool tap_ok = valid && tgi * KL + q < P.kV;
+                // Geometry, following the reference sampler (deform3d/lib/deform_conv3d_cuda_kernel.cu:21-26,
+                // 40-45,123-124) in a branch-free form: the coordinate is clamped into [0, size - 1];
+                // low corner = floor, fraction toward the high corner = clamped coordinate - floor.
+                // Where the reference collapses the high corner onto the low one (p <= 0,
+                // p >= size - 1) the fraction is 0, so the corner one step further carries weight 0
+                // and every sample uses the same eight (four) cells at fixed strides.
+                bool inside = tap_ok, inhalo = true;
+                T pq[ND], f[ND];
+                int u[ND];
+#pragma unroll
+                for (int a = 0; a < ND; ++a) {
+                    const int sa = slot<ND>(a);
+                    const T top = (T)(P.in[sa] - 1);
+                    const T pa = (ibf[a] + (T)(kq[a] * P.dil[sa])) + ofs[a];
+                    T pc;
+                    if constexpr (sizeof(T) == 4) pc = __builtin_amdgcn_fmed3f(pa, 0.f, top);
+                    else pc = fmin(fmax(pa, (T)0), top);
+                    const T fl = floor(pc);
+                    pq[a] = pa;
+                    f[a] = pc - fl;
+                    inside = inside && fabs(pa - pc) < (T)1;                // -1 < p < size, false for NaN
+                    u[a] = (int)fl - tg_.hb[a];
+                    inhalo = inhalo && (unsigned)u[a] < (unsigned)(P.hext[sa] - 1);
+                }
+                const bool near = inside && inhalo, far = inside && !inhalo;
+                unsigned base;
+                if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], P.hext[1]) + u[1], P.hext[2]) + u[2]);
+                else base = (unsigned)(__mul24(u[0], P.hext[2]) + u[1]);
+                base = near ? base : 0u;           // lanes without a sample in the halo read cell 0 and drop the value
+                T cw[NC];                          // corner weights, w_l * w_h * w_w
+                if constexpr (ND == 3) {
+                    const T fl = f[0], gl = (T)1 - fl, fh = f[1], gh = (T)1 - fh, fw = f[2], gw = (T)1 - fw;
+                    const T a00 = gl * gh, a01 = gl * fh, a10 = fl * gh, a11 = fl * fh;
+                    cw[0] = a00 * gw; cw[1] = a00 * fw; cw[2] = a01 * gw; cw[3] = a01 * fw;
+                    cw[4] = a10 * gw; cw[5] = a10 * fw; cw[6] = a11 * gw; cw[7] = a11 * fw;
+                } else {
+                    const T fh = f[0], gh = (T)1 - fh, fw = f[1], gw = (T)1 - fw;
+                    cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+                }
+                // next tap group's coordinates: KL single steps with carry, fastest axis last
+#pragma unroll
+                for (int st = 0; st < KL; ++st) {
+                    int carry = 1;
+#pragma unroll
+                    for (int a = ND - 1; a > 0; --a) {
+                        kq[a] += carry;
+                        carry = kq[a] >= P.k[slot<ND>(a)] ? 1 : 0;
+                        kq[a] = carry ? 0 : kq[a];
+                    }
+                    kq[0] += carry;
+                }
+                const V4* hp = reinterpret_cast<const V4*>(sIn) + base;
+                const T* wp = wchunk + (size_t)tgi * w_tg;
+                for (int grp = 0; grp < ngrp; ++grp) {
+                    V4 a4[MT];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) a4[mt] = *reinterpret_cast<const V4*>(wp + (w_lane + mt * w_tile));
+                    // weighted corner sum, four corners at a time (all eight in flight would cost 32
+                    // registers that the 16-wavefront shape does not have)
+                    // (element by element: a vector times scalar product would hold four copies of
+                    // every weight)
+                    T val[FQ];
+                    {
+                        V4 c4[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) c4[i] = hp[coff[i]];
+#pragma unroll
+                        for (int e = 0; e < FQ; ++e) {
+                            T v = c4[0][e] * cw[0];
+#pragma unroll
+                            for (int i = 1; i < 4; ++i) v += c4[i][e] * cw[i];
+                            val[e] = v;
+                        }
+                    }
+                    if constexpr (ND == 3) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        V4 c4[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) c4[i] = hp[coff[4 + i]];
+#pragma unroll
+                        for (int e = 0; e < FQ; ++e)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) val[e] += c4[i][e] * cw[4 + i];
+                    }
+#pragma unroll
+                    for (int e = 0; e < FQ; ++e) {
+                        const T b = near ? val[e] : (T)0;
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a4[mt][e], b, acc[mt]);
+                    }
+                    hp += P.hstride;
+                    wp += per_slab;
+                }
+                if (__any(far)) {                  // rare: some sample of this wave reaches past the halo
+                    TapGeo<T, ND> t;               // the reference's corner rule on the same coordinate
+                    t.inside = far;
+#pragma unroll
+                    for (int a = 0; a < ND; ++a) {
+                        const T pa = pq[a];
+                        const int l = far ? (int)pa : 0;
+                        t.p[a] = pa;
+                        t.lo[a] = l;
+                        t.hi[a] = (pa >= (T)(P.in[slot<ND>(a)] - 1) || pa <= (T)0) ? l : l + 1;
+                        t.f[a] = pa - (T)l;
+                    }
+                    tap_corner_idx<T, ND>(P, t);
+                    const T* wf = wchunk + (size_t)tgi * w_tg;
+                    for (int c = 0; c < nch; ++c) {
+                        T b = 0;
+                        if (far) b = sample<T, ND>(chan0 + (size_t)c * P.inV, t.idx, t.f);
+                        const T* wc = wf + (size_t)(c / FQ) * per_slab + c % FQ;
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wc[w_lane + mt * w_tile], b, acc[mt]);
+                    }
+                }
+            };
+            // two tap groups per trip: the offset registers of "this" and "next" swap roles without a
+            // copy (a copy would wait for the loads a whole tap group before they are needed)
+            for (int tgi = 0; tgi < ntg; tgi += 2) {
+                if (tgi + 1 < ntg) load_offsets_of(tgi + 1, o_buf[1]);
+                tap_group(tgi, o_buf[0]);
+                if (tgi + 1 < ntg) {
+                    if (tgi + 2 < ntg) load_offsets_of(tgi + 2, o_buf[0]);
+                    tap_group(tgi + 1, o_buf[1]);
+                }
+            }
+        }
+    }
+
+    if (!valid) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < MM::NACC; ++r) {
+            const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
+            if (m < P.M) {
+                T v = acc[mt][r];
+                if (bias) v += bias[g * P.M + m];
+                out[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+            }
+        }
+}
+
+}  // namespace dcn

@@ -97,7 +97,7 @@ def _geom(nd, inputs, weight, out_sizes, stride, padding, dilation, channel_per_
             list(weight.shape[2:]) + list(padding) + list(stride) + list(dilation) + [channel_per_group, group])
 
 
-def _workspace(inputs, weight, group, out_sizes):
+def _workspace(inputs, weight, group, out_sizes, channel_per_group):
     L = _lib.load()
     kV = inV = outV = 1
     for k in weight.shape[2:]:
@@ -106,8 +106,8 @@ def _workspace(inputs, weight, group, out_sizes):
         inV *= v
     for v in out_sizes:
         outV *= v
-    nbytes = L.dcn_workspace_bytes(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, outV,
-                                   kV, group)
+    nbytes = L.dcn_workspace_bytes_for(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, outV,
+                                       kV, group, channel_per_group)
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=inputs.device), int(nbytes)
 
 
@@ -128,7 +128,7 @@ def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channe
         _check(bias.dim() == 1 and bias.size(0) == weight.size(0), "bias size")
     inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
     output = torch.empty(out_shape, dtype=inputs.dtype, device=inputs.device)
-    ws, ws_bytes = _workspace(inputs, weight, group, outs)
+    ws, ws_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
     fn = getattr(L, "dcn%dd_forward_%s" % (nd, _SUFFIX[inputs.dtype]))
     with torch.cuda.device(inputs.device):
         rc = fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(),
@@ -152,7 +152,7 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
     suf = _SUFFIX[inputs.dtype]
     grad_input = grad_offset = grad_weight = None
     with torch.cuda.device(inputs.device):
-        ws, ws_bytes = _workspace(inputs, weight, group, outs)
+        ws, ws_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
         if need_data:
             # the kernels accumulate into grad_input (as the reference's atomicAdd does) and store
             # every element of grad_offset

@@ -67,6 +67,13 @@ const char *dcn_last_error(void);   /* message of the last failing call on this 
  * the backward calls, channels-last copies of the input batch, its gradient and grad_output. */
 size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
                            size_t output_volume, int kernel_volume, int group);
+/* The same for a known number of channels per deformable group (the reference's
+ * `channel_per_group`, deform3d/lib/deform_conv3d_cuda.cpp:66): never larger than the figure
+ * above, and much smaller for wide layers, whose per-chunk weight slabs the first query has to
+ * size for one-channel deformable groups.  0 for an inconsistent geometry. */
+size_t dcn_workspace_bytes_for(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
+                               size_t output_volume, int kernel_volume, int group,
+                               int channel_per_deformable_group);
 
 /* ---- 3-D, trilinear ------------------------------------------------------------------------
  * replaces deform3d/lib/deform_conv3d_cuda.cpp:90-165 (forward), :168-262 (backward_input_offset)
