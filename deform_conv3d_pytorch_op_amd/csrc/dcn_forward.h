@@ -78,8 +78,10 @@ __device__ inline void halo_stage_quads(const Params& P, const T* __restrict__ c
 
 // 1-D grid of N * tiles (3-D blocks of positions) * G * mchunks workgroups of NW wavefronts;
 // dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4 with cchunk a multiple of four.
+// (few accumulators: four wavefronts per SIMD, i.e. at most 128 registers, also for the 512-thread
+// shape, so that two of its workgroups share a CU)
 template <typename T, int ND, int MT, int NW>
-__global__ __launch_bounds__(NW * 64) void forward_quad_kernel(Params P, const T* __restrict__ in,
+__global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, const T* __restrict__ in,
                                                            const T* __restrict__ off, const T* __restrict__ Wq,
                                                            const T* __restrict__ bias, T* __restrict__ out) {
     using MM = Mma<T>;
