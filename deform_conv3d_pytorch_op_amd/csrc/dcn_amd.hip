@@ -202,7 +202,7 @@ static bool fused_chunk8() {      // DCN_FUSED_CHUNK=4: never take 8-channel chu
     return v != 0;
 }
 static int fused_first_waves() {
-    static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : (e && atoi(e) == 16) ? 16 : 8; }();
+    static const int v = [] { const char* e = getenv("DCN_FUSED_WAVES"); return (e && atoi(e) == 4) ? 4 : 8; }();
     return v;
 }
 static bool fused_fixed_stride() {      // DCN_FUSED_FIXED=0: runtime plane stride even where the compile-time one fits
@@ -463,11 +463,6 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
 #define DCN_LAUNCH_FUSED(BREG_, HS_, NW_) DCN_LAUNCH_FUSED_C(4, BREG_, HS_, NW_)
         if constexpr (ND == 2) {
             if (eight) return breg ? DCN_LAUNCH_FUSED_C(8, true, 0, 8) : DCN_LAUNCH_FUSED_C(8, false, 0, 8);
-        }
-        if (nw == 16) {      // experimental: 1024 threads, 8x8x8 positions, runtime plane stride
-            if (breg && !eight) { Ph.hstride = (Ph.hvol + 63) / 64 * 64; const size_t lds16 = (size_t)4 * Ph.hstride * (8 + sizeof(T)) + tables;
-                if (lds16 <= 160 * 1024) return launch_halo(backward_input_halo_kernel<T, ND, 4, true, true, 0, 16, true>, "backward_input_halo_kernel", hgrid, 1024, lds16, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit); }
-            continue;
         }
         if (nw == 8) {
             if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 8);

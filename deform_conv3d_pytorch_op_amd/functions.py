@@ -16,6 +16,8 @@ float32 and float64 are served by the same class for both 2-D and 3-D, and gradi
 not required come back as None instead of crashing (the reference wraps None in Variable, :76).
 All tensors must live on one MI355X; there is no CPU path.
 """
+import os
+
 import torch
 from torch.autograd import Function
 from torch.autograd.function import once_differentiable
@@ -115,6 +117,19 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+# backward_weight next to backward_input_offset on a second stream (DCN_OVERLAP_BACKWARD=0: one stream)
+_OVERLAP_BACKWARD = os.environ.get("DCN_OVERLAP_BACKWARD", "1") != "0"
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device):
+    """One extra stream per device, default priority, created on first use."""
+    key = torch.device(device).index
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)
+    return _SIDE_STREAMS[key]
+
+
 def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group, standard=False):
     L = _lib.load()
     stride, padding, dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
@@ -152,23 +167,38 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
     suf = _SUFFIX[inputs.dtype]
     grad_input = grad_offset = grad_weight = None
     with torch.cuda.device(inputs.device):
-        ws, ws_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
+        main = torch.cuda.current_stream()
+        # The two backward calls are independent.  When both are wanted, backward_weight runs on a
+        # second stream of the same priority with a workspace of its own: the fused kernel of
+        # backward_input_offset is bound by latencies and leaves room on every CU (LDS, registers,
+        # matrix and vector pipes) that the gathers of backward_weight fill.
+        side = _side_stream(inputs.device) if (need_data and need_weight and _OVERLAP_BACKWARD) else None
+        if need_weight:
+            grad_weight = torch.zeros_like(weight)          # beta = 1 accumulation, as in the reference
+            ws_w, ws_w_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
         if need_data:
+            ws, ws_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
             # the kernels accumulate into grad_input (as the reference's atomicAdd does) and store
             # every element of grad_offset
             grad_input = torch.zeros_like(inputs)
             grad_offset = torch.empty_like(offset)
+        if side is not None:
+            side.wait_stream(main)           # the operands and the zero fills above are ready
+        if need_data:
+            # issued first: its one large workgroup per CU takes its place and the small workgroups of
+            # backward_weight fill what is left, instead of the other way round
             args = (inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
-                    grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, _stream())
+                    grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, main.cuda_stream)
             if nd == 3 and oob_zero:        # the reference's 2-D kernels have no out-of-range term
                 _lib.check(getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)(*args, _lib.FLAG_OOB_OFFSET_GRAD_ZERO))
             else:
                 _lib.check(getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))(*args))
         if need_weight:
-            grad_weight = torch.zeros_like(weight)          # beta = 1 accumulation, as in the reference
             fn = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
             _lib.check(fn(inputs.data_ptr(), offset.data_ptr(), grad_output.data_ptr(), grad_weight.data_ptr(),
-                          *geom, ws.data_ptr(), ws_bytes, _stream()))
+                          *geom, ws_w.data_ptr(), ws_w_bytes, (side or main).cuda_stream))
+        if side is not None:
+            main.wait_stream(side)           # everything issued later on the caller's stream sees grad_weight
     return grad_input, grad_offset, grad_weight
 
 
