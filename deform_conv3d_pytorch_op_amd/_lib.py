@@ -51,6 +51,8 @@ def load():
             if nd == 3:
                 f = getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)
                 f.restype, f.argtypes = _c_int, [_c_vp] * 6 + geom + tail + [ctypes.c_uint]
+    L.dcn3d_forward_noalloc_f32.restype = _c_int
+    L.dcn3d_forward_noalloc_f32.argtypes = [_c_vp] * 5 + [_c_int] * N_GEOM[3] + [_c_vp]
     if L.dcn_version() != 1:
         raise ImportError("libdcn_amd.so has ABI version %d, expected 1" % L.dcn_version())
     _lib = L
@@ -65,5 +67,7 @@ def check(rc):
 EXPORTS = ["dcn_version", "dcn_arch", "dcn_last_error", "dcn_workspace_bytes", "dcn_workspace_bytes_for"] + [
     "dcn%dd_%s_%s" % (nd, op, suf)
     for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight") for suf in ("f32", "f64")] + [
-    "dcn3d_backward_input_offset_flags_f32", "dcn3d_backward_input_offset_flags_f64"]
+    "dcn3d_backward_input_offset_flags_f32", "dcn3d_backward_input_offset_flags_f64",
+    "dcn3d_forward_noalloc_f32"]
+NOALLOC_SCRATCH_BYTES = 8 << 20
 FLAG_OOB_OFFSET_GRAD_ZERO = 1

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 
 namespace {
@@ -657,6 +658,39 @@ Geometry geo2(int batch, int input_c, int output_c, int input_h, int input_w, in
                     {1, dilation_h, dilation_w}, cpg, group};
 }
 
+// ---------------------------------------------------------------------------------------------
+// Scratch of the allocation-free entry point: the re-laid-out weight of one forward call.  A
+// file-scope device array, so every GPU the library runs on holds DCN_NOALLOC_SCRATCH_BYTES of it
+// until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address is looked up once per device and kept, and host code
+// passes that address, never the name, to kernels.
+static __device__ __align__(256) unsigned char scratch[DCN_NOALLOC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+int scratch_address(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        (void)hipGetLastError();
+        return fail(DCN_E_DEVICE, "no current HIP device (or its ordinal is beyond 63)");
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            g_err = std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e);
+            return DCN_E_DEVICE;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return DCN_OK;
+}
+
 }  // namespace
 
 #define G3_ARGS batch, input_c, output_c, input_l, input_h, input_w, output_l, output_h, output_w, kernel_l, \
@@ -690,6 +724,29 @@ size_t dcn_workspace_bytes_for(int elem_size, int batch, int input_c, int output
     return elem_size == 8
                ? workspace_need<double>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg)
                : workspace_need<float>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg);
+}
+
+int dcn3d_forward_noalloc_f32(const float* input, const float* weight, const float* offset, const float* bias,
+                              float* output, DCN3D_GEOMETRY, void* stream) {
+    const Geometry g = geo3(G3_ARGS);
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    // what forward() asks of a workspace: either weight layout must fit the fixed array
+    int MT, mchunks, Mp, Cgp;
+    fwd_weight_pad<float>(P.M, P.Cg, MT, mchunks, Mp, Cgp);
+    const int Mp8 = ((P.M + 31) / 32 + 7) / 8 * 8 * 32;
+    const size_t plain = (size_t)P.G * P.kV * (Mp > Mp8 ? Mp : Mp8) * Cgp * sizeof(float);
+    const size_t quad = ((size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1) * forward_slab_elems<float>(P.kV, Mp8) * sizeof(float);
+    if (plain > DCN_NOALLOC_SCRATCH_BYTES || quad > DCN_NOALLOC_SCRATCH_BYTES) {
+        char msg[200];
+        snprintf(msg, sizeof msg, "layer too large for the allocation-free entry point: its re-laid-out weight takes %zu bytes, "
+                 "the fixed scratch holds %zu", plain > quad ? plain : quad, (size_t)DCN_NOALLOC_SCRATCH_BYTES);
+        return fail(DCN_E_WORKSPACE, msg);
+    }
+    void* ws = nullptr;
+    if (int rc = scratch_address(&ws)) return rc;
+    return forward<float, 3>(g, input, weight, offset, bias, output, ws, DCN_NOALLOC_SCRATCH_BYTES,
+                             static_cast<hipStream_t>(stream));
 }
 
 #define DEFINE_OPS(SUF, T)                                                                                          \

@@ -55,7 +55,7 @@ extern "C" {
 #define DCN_E_ARGUMENT   -1   /* inconsistent extents, null pointer, unsupported size */
 #define DCN_E_WORKSPACE  -2   /* workspace missing or too small */
 #define DCN_E_LAUNCH     -3   /* HIP reported an error when launching */
-#define DCN_E_DEVICE     -4   /* current device is not a gfx950 GPU */
+#define DCN_E_DEVICE     -4   /* no current HIP device, or a query of it failed */
 
 int dcn_version(void);              /* ABI version, currently 1 */
 const char *dcn_arch(void);         /* the code-object target the kernels were built for: "gfx950" */
@@ -97,6 +97,19 @@ int dcn3d_backward_input_offset_f32(const float *input, const float *weight, con
 int dcn3d_backward_input_offset_f64(const double *input, const double *weight, const double *offset,
                                     const double *grad_output, double *grad_input, double *grad_offset,
                                     DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Forward pass that allocates nothing and takes no workspace.  No counterpart in the reference: it
+ * is for callers that cannot allocate device memory around the call (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  Same arguments, results and kernels as
+ * dcn3d_forward_f32 without the workspace pair; the re-laid-out weight goes into a fixed device array
+ * of DCN_NOALLOC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until
+ * the process ends.  A layer whose re-laid-out weight is larger (roughly: 4 * kernel volume *
+ * output_c rounded up to 256 * (input_c / group + 4) bytes) is rejected with DCN_E_WORKSPACE.  All
+ * calls on one GPU share that array: calls that overlap there (two streams, two threads) race on it
+ * and must be serialised by the caller; calls on different GPUs are independent. */
+#define DCN_NOALLOC_SCRATCH_BYTES (8u << 20)
+int dcn3d_forward_noalloc_f32(const float *input, const float *weight, const float *offset, const float *bias,
+                              float *output, DCN3D_GEOMETRY, void *stream);
 
 /* The same call with option flags.  No counterpart in the reference, whose 3-D col2im_offset kernel
  * always adds +-|grad column| to grad_offset for a sample that lies outside the input
