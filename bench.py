@@ -1,14 +1,15 @@
 """Benchmark of the deformable-convolution hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c4] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5|all] [--no-cpu]
 
 A step is one forward + backward (grad input, grad offset, grad weight) of one layer through the
 package's autograd Function on synthetic inputs already resident in HBM.  The default workload is
 BASELINE.json's headline configuration c4: deform3d float32, N=4, 64->64 channels, 16x56x56,
 kernel 3x3x3, stride 1, pad 1, one deformable group, offsets U[-1.5, 1.5].
 
-Prints one JSON line.  `value` is effective TFLOP/s = 3 * 2*N*C_out*(C_in/G)*kV*outV / step time
-(only the three dense contractions are counted as work).  `roofline` describes the slowest kernel
+Prints one JSON line (`--config all`: one line per configuration, c1 to c5).  `value` is effective
+TFLOP/s = 3 * 2*N*C_out*(C_in/G)*kV*outV / step time (only the three dense contractions are counted
+as work).  `roofline` describes the slowest kernel
 of the step, timed on its own with HIP events on the stream it is launched on; `cpu_baseline` is
 the CPU oracle (the reference algorithm restated: im2col + GEMM per sample and group) timed on a
 bounded sample of the same workload on the host cores.
@@ -29,14 +30,20 @@ PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}     # MI355X dense matrix peak
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch measured with rocprofv3 (--pmc FETCH_SIZE, then --pmc WRITE_SIZE, each scaled by
-# what the same counter reads for a plain 256 MiB device copy in the same run: 2.0 and 1.0 KiB per unit);
-# the summary with the commands is profiles/c4_deform3d_f32_fwd_bwd_kernels.md.  Only for configurations
-# that were profiled; otherwise `traffic` is null.
-MEASURED_TRAFFIC_BYTES = {
-    ("c4", "forward"): 0.524e9,
-    ("c4", "backward_input_offset"): 1.992e9,
-    ("c4", "backward_weight"): 1.211e9,
-}
+# what the same counter reads for a plain 256 MiB device copy in the same run).  The figures live in a data
+# file that is rewritten whenever the kernels are profiled again: {"c4": {"forward": bytes, ...}, ...}.
+# A configuration or call that was not profiled has no entry and reports `traffic` null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(config, call):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            v = json.load(f).get(config, {}).get(call)
+        return float(v) if v is not None else None
+    except (OSError, ValueError):
+        return None
+
 
 # name: (nd, N, C_in, C_out, in, k, stride, pad, dil, cpg, groups, offset scale / dist, dtype)
 CONFIGS = {
@@ -71,27 +78,14 @@ def algorithmic_bytes(c):
     return dict(forward=fwd, backward_input_offset=data, backward_weight=wgt)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="c4", choices=sorted(CONFIGS))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 256 MiB device copy (a kernel of known traffic for scaling rocprof's "
-                         "FETCH_SIZE / WRITE_SIZE counters)")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
-
+def run_config(name, a):
     import torch
     import deform_conv3d_pytorch_op_amd as dcn
     from deform_conv3d_pytorch_op_amd import _lib
     from deform_conv3d_pytorch_op_amd.functions import _geom
     from tests.cases import make_case
 
-    spec = CONFIGS[a.config]
+    spec = CONFIGS[name]
     dtype = getattr(torch, spec[-1])
     kw = dict(dtype=dtype, seed=0, bias=False)
     if spec[-2] == "normal_mix":
@@ -151,8 +145,8 @@ def main():
     L = _lib.load()
     suf = "f32" if dtype == torch.float32 else "f64"
     geom = _geom(nd, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
-    nbytes = L.dcn_workspace_bytes(x.element_size(), x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]),
-                                   math.prod(c["outs"]), math.prod(c["k"]), c["groups"])
+    nbytes = L.dcn_workspace_bytes_for(x.element_size(), x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]),
+                                       math.prod(c["outs"]), math.prod(c["k"]), c["groups"], c["cpg"])
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     out = torch.empty((x.shape[0], w.shape[0]) + c["outs"], dtype=dtype, device=dev)
     gin, goff, gw = torch.zeros_like(x), torch.empty_like(off), torch.zeros_like(w)
@@ -169,7 +163,7 @@ def main():
             xd.data_ptr(), od.data_ptr(), gout.data_ptr(), gw.data_ptr(), *geom, ws.data_ptr(), nbytes, sp),
     }
     kernel_ms = {}
-    for name, call in calls.items():
+    for cname, call in calls.items():
         for _ in range(2):
             assert call() == 0, L.dcn_last_error()
         evs = []
@@ -180,14 +174,14 @@ def main():
             e1.record(stream)
             evs.append((e0, e1))
         torch.cuda.synchronize()
-        kernel_ms[name] = sum(e0.elapsed_time(e1) for e0, e1 in evs) / len(evs)
+        kernel_ms[cname] = sum(e0.elapsed_time(e1) for e0, e1 in evs) / len(evs)
     dominant = max(kernel_ms, key=kernel_ms.get)
     ab = algorithmic_bytes(c)
     peak = PEAK_TFLOPS[spec[-1]]
     achieved = F / (kernel_ms[dominant] * 1e-3) / 1e12
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": round(achieved, 3), "peak": peak,
                 "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get((a.config, dominant)),
+                "traffic": measured_traffic(name, dominant),
                 "ms": round(kernel_ms[dominant], 4),
                 "algorithmic_flops": F, "algorithmic_bytes": ab[dominant],
                 "hbm_frac_at_algorithmic_bytes": round(ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
@@ -207,29 +201,49 @@ def main():
         from oracle import dcn_oracle as orc
         ns = x.shape[0]
         xs, offs, gs = c["x"][:ns].contiguous(), c["off"][:ns].contiguous(), c["gout"][:ns].contiguous()
-        reps, times = 9, []
-        for _ in range(reps):                  # about 12 s of host work at c4 (16 threads)
+        def once():
             t0 = time.perf_counter()
             orc.forward(xs, offs, c["w"], None, *cfg, acc64=False)
             orc.backward(xs, offs, c["w"], gs, None, *cfg, acc64=False)
-            times.append(time.perf_counter() - t0)
+            return time.perf_counter() - t0
+        first = once()                         # also warms the thread pool; not counted
+        reps = max(3, min(25, int(12.0 / max(first, 1e-3))))      # about 12 s of host work per configuration
+        times = [once() for _ in range(reps)]
         dt = sorted(times)[len(times) // 2]
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
         cpu = {"value": round(3 * F * ns / x.shape[0] / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
                "kind": "port", "seconds": round(dt, 2),
                "sample": "%d of %d samples of %s, forward + backward, median of %d runs, float accumulate, OpenMP" %
-                         (ns, x.shape[0], a.config, reps)}
+                         (ns, x.shape[0], name, reps)}
 
-    print(json.dumps({
+    return {
         "metric": "deform conv fwd+bwd effective TFLOP/s per layer (3 dense contractions counted)",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_step, 4), "fwd_ms": round(ms_fwd, 4),
         "ms_per_step_events": step_events, "fwd_ms_events": fwd_events, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32" if dtype == torch.float32 else "f64", "data": "synthetic",
-        "config": {"workload": a.config + ": " + DESCR[a.config]},
+        "config": {"workload": name + ": " + DESCR[name]},
         "mfma_frac_whole_step": round(value / peak, 4),
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
-    }))
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c4", choices=sorted(CONFIGS) + ["all"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic for scaling rocprof's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    for name in (sorted(CONFIGS) if a.config == "all" else [a.config]):
+        print(json.dumps(run_config(name, a)), flush=True)
 
 
 if __name__ == "__main__":

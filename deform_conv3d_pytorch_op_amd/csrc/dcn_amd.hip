@@ -8,8 +8,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <string>
+#include <utility>
 
 namespace {
 
@@ -180,16 +182,38 @@ static bool fused_coord() {
     static const int v = [] { const char* e = getenv("DCN_COORD"); return (e && strcmp(e, "separate") == 0) ? 0 : 1; }();
     return v != 0;
 }
-static int cu_count() {
-    static const int v = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+// What the library needs to know about a GPU, looked up once per device ordinal.
+struct DeviceInfo { int state = 0; int cus = 256; };      // state: 0 not looked up, 1 usable, -1 not a gfx950
+constexpr int MAX_DEVICES = 64;
+std::mutex g_device_lock;
+DeviceInfo g_device[MAX_DEVICES];
+
+// Fills `out` for the current device; DCN_E_DEVICE when there is none or it is not a gfx950.
+int device_info(const DeviceInfo** out, int* ordinal = nullptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        (void)hipGetLastError();
+        return fail(DCN_E_DEVICE, "no current HIP device (or its ordinal is beyond 63)");
+    }
+    std::lock_guard<std::mutex> lock(g_device_lock);
+    DeviceInfo& d = g_device[dev];
+    if (d.state == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
             (void)hipGetLastError();
-            n = 256;
+            return fail(DCN_E_DEVICE, "hipGetDeviceProperties failed");
         }
-        return n;
-    }();
-    return v;
+        d.state = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+        if (prop.multiProcessorCount > 0) d.cus = prop.multiProcessorCount;
+    }
+    if (d.state < 0) return fail(DCN_E_DEVICE, "the current device is not a gfx950 GPU");
+    if (out) *out = &d;
+    if (ordinal) *ordinal = dev;
+    return DCN_OK;
+}
+static int cu_count() {      // of the current device (every entry point has called device_info by then)
+    const DeviceInfo* d = nullptr;
+    return device_info(&d) == DCN_OK ? d->cus : 256;
 }
 static int wide_forward() {      // 0 never, 1 when it pays, 2 whenever the halo fits
     static const int v = [] {
@@ -215,15 +239,17 @@ static bool scatter_in_lds() {
     return v != 0;
 }
 #define LDS_BUDGET lds_budget()
-int g_halo_margin = -1;                          // test hook: DCN_HALO_MARGIN overrides the default of 2
-
-int halo_margin() {
-    if (g_halo_margin < 0) {
+static int halo_margin() {      // DCN_HALO_MARGIN overrides the default of 2 voxels
+    static const int v = [] {
         const char* e = getenv("DCN_HALO_MARGIN");
-        g_halo_margin = e ? atoi(e) : 2;
-        if (g_halo_margin < 0) g_halo_margin = 0;
-    }
-    return g_halo_margin;
+        const int m = e ? atoi(e) : 2;
+        return m < 0 ? 0 : m;
+    }();
+    return v;
+}
+static int forced_csplit() {    // DCN_CSPLIT=n: workgroups per (tile, deformable group) of the fused backward kernel
+    static const int v = [] { const char* e = getenv("DCN_CSPLIT"); return e && atoi(e) > 0 ? atoi(e) : 0; }();
+    return v;
 }
 
 template <typename T, int ND>
@@ -277,15 +303,28 @@ bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_by
     return true;
 }
 
+// Raises a kernel's dynamic LDS limit; the runtime is asked only when a kernel needs more than it
+// was last granted on the current device.
+int raise_lds_limit(const void* kern, size_t lds) {
+    static std::mutex lock;
+    static std::map<std::pair<int, const void*>, size_t> granted;
+    int dev = 0;
+    if (device_info(nullptr, &dev) != DCN_OK) return DCN_E_DEVICE;
+    std::lock_guard<std::mutex> guard(lock);
+    size_t& have = granted[std::make_pair(dev, kern)];
+    if (lds <= have) return DCN_OK;
+    if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
+    }
+    have = lds;
+    return DCN_OK;
+}
+
 template <typename K, typename... Args>
 int launch_halo(K kern, const char* name, dim3 grid, int threads, size_t lds, hipStream_t s, Args... args) {
-    if (lds > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
-        }
-    }
+    if (lds > 48 * 1024)
+        if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return rc;
     hipLaunchKernelGGL(kern, grid, dim3(threads), lds, s, args...);
     return check_launch(name);
 }
@@ -296,6 +335,7 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (!in || !w || !off || !out) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    if (int rc = device_info(nullptr)) return rc;
     int MT;
     fwd_weight_pad<T>(P.M, P.Cg, MT, P.mchunks, P.Mp, P.Cgp);
     if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
@@ -363,6 +403,8 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     // geometry whose halo does not fit in LDS: gather straight from global memory
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
+    if ((long long)P.N * P.tiles > 0x7fffffffLL || (long long)P.G * P.mchunks > 65535)
+        return fail(DCN_E_ARGUMENT, "layer too large for the kernel without LDS tiling (groups x output-channel chunks > 65535)");
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.G * P.mchunks);
     switch (MT) {
         case 1: hipLaunchKernelGGL((forward_kernel<T, ND, 1>), grid, dim3(WG), 0, s, P, in, off, wt, bias, out); break;
@@ -388,6 +430,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (flags & ~(unsigned)DCN_FLAG_OOB_OFFSET_GRAD_ZERO) return fail(DCN_E_ARGUMENT, "unknown flag");
+    if (int rc = device_info(nullptr)) return rc;
     P.oob_zero = (flags & DCN_FLAG_OOB_OFFSET_GRAD_ZERO) ? 1 : 0;
     if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     bwd_data_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
@@ -445,7 +488,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             const double rounds = (double)((items * cs + cus - 1) / cus) / cs;
             if (rounds < best * 0.97) { best = rounds; csplit = cs; }
         }
-        if (const char* e = getenv("DCN_CSPLIT")) csplit = atoi(e) > 0 ? atoi(e) : csplit;
+        if (forced_csplit()) csplit = forced_csplit();
         if (csplit > nchunks) csplit = nchunks;
         if (csplit > 1) {
             const size_t nel = (size_t)P.N * P.DG * P.kV * ND * P.outV;
@@ -496,6 +539,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         else halo = false;
     }
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
+    if ((long long)P.N * P.tiles > 0x7fffffffLL || P.DG > 65535)
+        return fail(DCN_E_ARGUMENT, "layer too large for the kernel without the fused LDS halo (more than 65535 deformable groups)");
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
     if (halo) {
         T* none = nullptr;
@@ -583,13 +628,8 @@ int launch_bwd_weight(const Params& P, const T* in_cl, const T* off, const T* go
     const int TN = Mma<T>::TN;
     const size_t lds = (size_t)WAVES * TN * (TN + 1) * sizeof(T);
     auto kern = backward_weight_kernel<T, ND, MT>;
-    if (lds > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(DCN_E_LAUNCH, "cannot raise the dynamic LDS limit");
-        }
-    }
+    if (lds > 48 * 1024)
+        if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return rc;
     const dim3 grid((unsigned)P.nsplit * P.kV * P.nctiles * P.mchunks);
     hipLaunchKernelGGL(kern, grid, dim3(WG), lds, s, P, in_cl, off, gout_cl, partial);
     return check_launch("backward_weight_kernel");
@@ -607,6 +647,7 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    if (int rc = device_info(nullptr)) return rc;
     if ((long long)P.outV * P.C_out > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one output sample exceeds 2^31 elements");
     // the kernel addresses both operands by 32-bit byte offsets from the sample's base
     if ((unsigned long long)P.inV * P.C_in * sizeof(T) >= (1ull << 32) || (unsigned long long)P.outV * P.C_out * sizeof(T) >= (1ull << 32))
@@ -615,7 +656,7 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     bww_plan<T>(P, MT, P.mchunks, P.nctiles, P.nsplit);
     const long long resident = MT == 1 ? bww_resident<T, ND, 1>() : MT == 2 ? bww_resident<T, ND, 2>() : bww_resident<T, ND, 4>();
     bww_plan<T>(P, MT, P.mchunks, P.nctiles, P.nsplit, resident);
-    if ((long long)P.nctiles * P.mchunks > 65535) return fail(DCN_E_ARGUMENT, "too many channel tiles for one launch");
+    if ((long long)P.nsplit * P.kV * P.nctiles * P.mchunks > 0x7fffffffLL) return fail(DCN_E_ARGUMENT, "too many workgroups for one launch");
     const size_t ibytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
     const size_t obytes = align256((size_t)P.N * P.C_out * P.outV * sizeof(T));
     if (!ws || ws_bytes < bww_workspace<T>(P, P.nsplit)) return fail(DCN_E_WORKSPACE, "workspace too small");
@@ -666,16 +707,12 @@ Geometry geo2(int batch, int input_c, int output_c, int input_h, int input_w, in
 // passes that address, never the name, to kernels.
 static __device__ __align__(256) unsigned char scratch[DCN_NOALLOC_SCRATCH_BYTES];
 
-constexpr int MAX_DEVICES = 64;
 std::mutex g_scratch_lock;
 void* g_scratch_ptr[MAX_DEVICES] = {};
 
 int scratch_address(void** out) {
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
-        (void)hipGetLastError();
-        return fail(DCN_E_DEVICE, "no current HIP device (or its ordinal is beyond 63)");
-    }
+    if (int rc = device_info(nullptr, &dev)) return rc;
     std::lock_guard<std::mutex> lock(g_scratch_lock);
     if (!g_scratch_ptr[dev]) {
         void* p = nullptr;
