@@ -171,6 +171,10 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
 //   DCN_FUSED_WAVES=4      fused backward kernel with four wavefronts per workgroup even where eight fit
 //   DCN_FUSED_CHUNK=4      fused backward kernel with 4-channel chunks also where it would take 8 (2-D layers)
+//   DCN_FUSED_TAIL=0       fused backward kernel: all items split alike, never only those of the last round
+//   DCN_CSPLIT=n           fused backward kernel: every item split over n workgroups
+//   DCN_FUSED_SLOTS=n      fused backward kernel: plan the launch as if n workgroups ran at once (test hook)
+//   DCN_FUSED_FIXED=0      fused backward kernel: runtime plane stride even where the compile-time one fits
 static size_t env_kb(const char* name, int dflt) {
     const char* e = getenv(name);
     const int v = e ? atoi(e) : dflt;
@@ -233,6 +237,14 @@ static int fused_first_waves() {
 static bool fused_fixed_stride() {      // DCN_FUSED_FIXED=0: runtime plane stride even where the compile-time one fits
     static const int v = [] { const char* e = getenv("DCN_FUSED_FIXED"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
+}
+static bool fused_tail_split() {        // DCN_FUSED_TAIL=0: the fused backward kernel never splits only the items of the last round
+    static const int v = [] { const char* e = getenv("DCN_FUSED_TAIL"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
+}
+static int forced_slots() {             // DCN_FUSED_SLOTS=n (test hook): plan the fused backward launch as if n workgroups ran at once
+    static const int v = [] { const char* e = getenv("DCN_FUSED_SLOTS"); return e && atoi(e) > 0 ? atoi(e) : 0; }();
+    return v;
 }
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
@@ -319,6 +331,25 @@ int raise_lds_limit(const void* kern, size_t lds) {
     }
     have = lds;
     return DCN_OK;
+}
+
+// Workgroups of a kernel that the current device holds at once (one per CU if the query fails).
+long long resident_workgroups(const void* kern, int threads, size_t lds) {
+    static std::mutex lock;
+    static std::map<std::pair<const void*, size_t>, int> per_cu_of;
+    int per_cu = 0;
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        int& v = per_cu_of[std::make_pair(kern, lds)];
+        if (v == 0) {
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, kern, threads, lds) != hipSuccess || v < 1) {
+                (void)hipGetLastError();
+                v = 1;
+            }
+        }
+        per_cu = v;
+    }
+    return (long long)per_cu * cu_count();
 }
 
 template <typename K, typename... Args>
@@ -477,47 +508,67 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
-        // split the channel chunks of a (tile, deformable group) over 1, 2 or 4 workgroups, whichever
-        // wastes least of the last round (one workgroup per CU at this LDS size)
+        // grad_output operand held in registers when its reduction steps fit: 8 per tap slot of a pass
+        // (M <= 64 float, 128 double with 4-channel chunks)
+        const int slot_regs = (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
+        const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= Mma<T>::NACC / slot_regs * 8;
+        using Kern = void (*)(Params, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
+        Kern kern = nullptr;
+#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true>
+#define DCN_FUSED(BREG_, HS_, NW_) DCN_FUSED_C(4, BREG_, HS_, NW_)
+        if constexpr (ND == 2) {
+            if (eight) kern = breg ? DCN_FUSED_C(8, true, 0, 8) : DCN_FUSED_C(8, false, 0, 8);
+        }
+        if (!kern) {
+            if (nw == 8) kern = fixed && breg ? DCN_FUSED(true, FUSED_HS, 8) : fixed ? DCN_FUSED(false, FUSED_HS, 8) : DCN_FUSED(false, 0, 8);
+            else kern = fixed && breg ? DCN_FUSED(true, FUSED_HS, 4) : fixed ? DCN_FUSED(false, FUSED_HS, 4) : DCN_FUSED(false, 0, 4);
+        }
+#undef DCN_FUSED
+#undef DCN_FUSED_C
+        if (lds > 48 * 1024)
+            if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return rc;
+        // Work items are (tile, deformable group) pairs, each a run of nchunks channel chunks.  `slots`
+        // workgroups run at once, so the items take whole rounds plus a partly filled last one.  Either
+        // every item is split over 1, 2 or 4 workgroups (workgroup cz takes every csplit-th chunk), or
+        // the items of the whole rounds stay unsplit and only those of the last round are split, as
+        // finely as fills the device; they come last in the launch.  A workgroup's fixed part
+        // (grad_output operand, halo table, offsets) costs about a quarter of a chunk, which the
+        // estimate charges per split.  The chunks of an item add their grad_offset parts with float
+        // atomics on a zero-filled buffer (measured faster than read-modify-write by one workgroup);
+        // an item of a single chunk stores.
         const int nchunks = (seg + cch - 1) / cch;
         const long long items = (long long)Ph.N * Ph.tiles * Ph.DG;
-        const int cus = cu_count();
+        const long long slots = forced_slots() ? forced_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
+        auto item_cost = [&](double chunks_per_wg, int wgs) { return wgs * (chunks_per_wg + 0.25) / nchunks; };
         int csplit = 1;
+        long long whole = 0;                              // unsplit items at the start of the launch
         double best = 1e30;
         for (int cs = 1; cs <= 4 && cs <= nchunks; cs *= 2) {
-            const double rounds = (double)((items * cs + cus - 1) / cus) / cs;
-            if (rounds < best * 0.97) { best = rounds; csplit = cs; }
+            const double rounds = (double)((items * cs + slots - 1) / slots) / cs * item_cost((double)nchunks / cs, cs);
+            if (rounds < best) { best = rounds; csplit = cs; }
         }
-        if (forced_csplit()) csplit = forced_csplit();
+        if (fused_tail_split() && items > slots && items % slots) {
+            const long long rest = items % slots;
+            const long long cs = slots / rest < nchunks ? slots / rest : nchunks;
+            if (cs >= 2) {
+                const double rounds = (double)(items / slots) * item_cost(nchunks, 1) + item_cost((double)((nchunks + cs - 1) / cs), 1);
+                if (rounds < best) { best = rounds; csplit = (int)cs; whole = items - rest; }
+            }
+        }
+        if (forced_csplit()) { csplit = forced_csplit(); whole = 0; }
         if (csplit > nchunks) csplit = nchunks;
-        if (csplit > 1) {
+        const int goff_atomic = nchunks > 1 ? 1 : 0;
+        if (goff_atomic) {
             const size_t nel = (size_t)P.N * P.DG * P.kV * ND * P.outV;
             const unsigned fb = (unsigned)((nel + 1023) / 1024 > 8192 ? 8192 : (nel + 1023) / 1024);
             hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fb), dim3(256), 0, s, goff, nel);
             if (int rc = check_launch("fill_zero_kernel")) return rc;
         }
-        const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG * csplit);
-        // grad_output operand held in registers when its reduction steps fit: 8 per tap slot of a pass
-        // (M <= 64 float, 128 double with 4-channel chunks)
-        const int slot_regs = (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
-        const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= Mma<T>::NACC / slot_regs * 8;
-#define DCN_LAUNCH_FUSED_C(CCH_, BREG_, HS_, NW_)                                                                     \
-    launch_halo(backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true>, "backward_input_halo_kernel", hgrid, NW_ * 64, \
-                lds, s, Ph, in, off, wt, gout, wmax, gin, goff, csplit)
-#define DCN_LAUNCH_FUSED(BREG_, HS_, NW_) DCN_LAUNCH_FUSED_C(4, BREG_, HS_, NW_)
-        if constexpr (ND == 2) {
-            if (eight) return breg ? DCN_LAUNCH_FUSED_C(8, true, 0, 8) : DCN_LAUNCH_FUSED_C(8, false, 0, 8);
-        }
-        if (nw == 8) {
-            if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 8);
-            if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 8);
-            return DCN_LAUNCH_FUSED(false, 0, 8);
-        }
-        if (fixed && breg) return DCN_LAUNCH_FUSED(true, FUSED_HS, 4);
-        if (fixed) return DCN_LAUNCH_FUSED(false, FUSED_HS, 4);
-        return DCN_LAUNCH_FUSED(false, 0, 4);
-#undef DCN_LAUNCH_FUSED
-#undef DCN_LAUNCH_FUSED_C
+        if (whole + (items - whole) * csplit > 0x7fffffffLL) return fail(DCN_E_ARGUMENT, "too many workgroups for one launch");
+        hipLaunchKernelGGL(kern, dim3((unsigned)(whole + (items - whole) * csplit)), dim3(nw * 64), lds, s, Ph, in, off, wt, gout,
+                           wmax, gin, goff, csplit, (unsigned)whole, goff_atomic);
+        if (int rc = check_launch("backward_input_halo_kernel")) return rc;
+        return DCN_OK;
     }
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
@@ -557,10 +608,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         T* nogoff = nullptr;
         if (Ph.cchunk == 8)
             return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false, 0, WAVESH>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
-                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1);
+                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1, 0u, 0);
         if (Ph.cchunk == 4)
             return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false, 0, WAVESH>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
-                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1);
+                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1, 0u, 0);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }
     // halo does not fit in LDS: scatter with global atomics on the channels-last copy

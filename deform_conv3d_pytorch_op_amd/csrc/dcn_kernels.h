@@ -851,14 +851,15 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // After all taps the planes are added to grad_input with one hardware float atomic per touched
 // halo voxel -- about 1/30 of the global atomics of a direct scatter.  Samples that reach past
 // the halo use global atomics directly, in a pass of their own.
-// 1-D grid of DG * N * tiles * csplit workgroups; dynamic LDS = CCH * hstride * 8 + hvol * 4 +
-// kV * ND * 4 bytes.
+// 1-D grid: `whole` workgroups with one (tile, deformable group) item each, then csplit
+// workgroups for each remaining item; dynamic LDS = CCH * hstride * 8 + hvol * 4 bytes.
 // COORD = true additionally stages the same CCH input channels over the halo (float planes) and
 // computes grad_offset in the same pass over the grad-column values (col2im_offset of the
 // reference, deform3d kernel.cu:386-483 incl. the out-of-range branches :470-481, 2-D
 // deform2d_double kernel.cu:309-366): per (tap, position) the derivative of the interpolation
 // along each axis times gcol, summed over the chunk's channels, accumulated into grad_offset
-// chunk after chunk (the first chunk stores).  dynamic LDS then adds CCH * hstride * sizeof(T).
+// chunk after chunk (float atomics on a zero-filled buffer, or the first chunk stores and the
+// others add in place).  dynamic LDS then adds CCH * hstride * sizeof(T).
 // BREG = true (host: at most NS * 8 reduction steps, i.e. M <= 64 for float) keeps this lane's
 // grad_output values -- the B operand, the same for every tap and channel chunk -- in registers.
 // NW wavefronts per workgroup (8; 4 where only a smaller block of positions has a halo that fits).
@@ -872,7 +873,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                                                                   const T* __restrict__ Wt,
                                                                   const T* __restrict__ gout,
                                                                   const float* __restrict__ wmax,
-                                                                  T* __restrict__ gin, T* __restrict__ goff, int csplit) {
+                                                                  T* __restrict__ gin, T* __restrict__ goff, int csplit,
+                                                                  unsigned whole, int goff_atomic) {
     using MM = Mma<T>;
     using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
@@ -889,17 +891,26 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     __shared__ float sRed[NW];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
-    // 1-D grid of DG * N * tiles * csplit workgroups.  csplit workgroups share one (tile, deformable
-    // group): workgroup cz takes every csplit-th channel chunk (finer work items shorten the last,
-    // partly filled round of workgroups).  Their grad_offset contributions then meet through float
-    // atomics on a zero-filled buffer.
-    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
-    const int cz = wg % (unsigned)csplit;
+    // Work items are (tile, deformable group) pairs.  The first `whole` workgroups of the launch take
+    // one item each; every later item is shared by csplit workgroups, of which workgroup cz takes
+    // every csplit-th channel chunk: finer work at the end of the launch fills the last, ragged
+    // round of workgroups.  goff_atomic: the grad_offset contributions of the channel chunks meet
+    // through float atomics on a zero-filled buffer (required where an item is shared); otherwise
+    // the first chunk stores and later ones add in place.
+    unsigned item;
+    int cz = 0, cs = 1;
+    if (blockIdx.x < whole) item = xcd_contiguous(blockIdx.x, whole);
+    else {
+        const unsigned r = xcd_contiguous(blockIdx.x - whole, gridDim.x - whole);
+        cs = csplit;
+        item = whole + r / (unsigned)cs;
+        cz = r % (unsigned)cs;
+    }
     const unsigned nt = (unsigned)P.N * P.tiles;
-    const int dg = (wg / csplit) / nt;
+    const int dg = item / nt;
 
     TileGeo<ND> tg;
-    tile_decode<ND>(P, (wg / csplit) % nt, tg);
+    tile_decode<ND>(P, item % nt, tg);
     const int n = tg.n;
     int o[ND], ib[ND];
     unsigned pos;
@@ -916,7 +927,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
     const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
     T* goff_dg = goff + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
-    bool first_chunk = true;                        // grad_offset (csplit == 1): the first channel chunk stores, later ones add
+    bool first_chunk = true;                        // grad_offset without atomics: the first channel chunk stores, later ones add
     int chunk_no = 0;
     // this lane's row of the A operand: (tap slot, channel) = (j / CCH, j % CCH)
     const int a_tl = j / CCH, a_c = j % CCH;
@@ -1000,7 +1011,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         const double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
 
         for (int cc0 = rb; cc0 < re; cc0 += CCH) {
-            if ((chunk_no++) % csplit != cz) continue;          // another workgroup's chunk (uniform)
+            if ((chunk_no++) % cs != cz) continue;          // another workgroup's chunk (uniform)
             const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < nch; ++c)
@@ -1141,7 +1152,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     T* gp = goff_dg + (size_t)pend_tap * ND * P.outV + pos;
 #pragma unroll
                     for (int a = 0; a < ND; ++a) {
-                        if (csplit > 1) { if (pend_ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, pend_ga[a]); }
+                        if (goff_atomic) { if (pend_ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, pend_ga[a]); }
                         else if (first_chunk) gp[(size_t)a * P.outV] = pend_ga[a];
                         else gp[(size_t)a * P.outV] += pend_ga[a];
                     }

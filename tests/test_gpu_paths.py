@@ -11,6 +11,10 @@ settings, each in a process of its own (the knobs are read once per process):
   DCN_CSPLIT=1 / 4     channel chunks of the fused backward kernel on one / four workgroups
   DCN_FUSED_WAVES=4    the fused backward kernel's four-wavefront shape (otherwise only strided full-size cases use it)
   DCN_FUSED_CHUNK=4    the fused backward kernel with 4-channel chunks also for 2-D layers (which otherwise take 8)
+  DCN_FUSED_SLOTS=3    plans the fused backward launch for a device of three workgroups: unsplit items first, the
+                       items of the last round split over several workgroups (otherwise only full-size layers get there)
+  DCN_FUSED_TAIL=0     ... and the same without that split; DCN_FUSED_FIXED=0: runtime plane stride
+  DCN_OVERLAP_BACKWARD=1  backward_weight on a second stream next to backward_input_offset
 """
 import os
 import subprocess
@@ -31,6 +35,9 @@ SETTINGS = [
     {"DCN_COORD": "separate"},
     {"DCN_FUSED_WAVES": "4"},
     {"DCN_FUSED_CHUNK": "4"},
+    {"DCN_FUSED_SLOTS": "3"},
+    {"DCN_FUSED_SLOTS": "3", "DCN_FUSED_TAIL": "0", "DCN_FUSED_FIXED": "0"},
+    {"DCN_OVERLAP_BACKWARD": "1"},
 ]
 
 
