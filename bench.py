@@ -16,6 +16,7 @@ bounded sample of the same workload on the host cores.
 """
 import argparse
 import ctypes
+import hashlib
 import json
 import math
 import os
@@ -29,17 +30,31 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}     # MI355X dense matrix peaks
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 (--pmc FETCH_SIZE, then --pmc WRITE_SIZE, each scaled by
+# HBM bytes per C-ABI call measured with rocprofv3 (--pmc FETCH_SIZE, then --pmc WRITE_SIZE, each scaled by
 # what the same counter reads for a plain 256 MiB device copy in the same run).  The figures live in a data
-# file that is rewritten whenever the kernels are profiled again: {"c4": {"forward": bytes, ...}, ...}.
-# A configuration or call that was not profiled has no entry and reports `traffic` null.
+# file that is rewritten whenever the kernels are profiled again: {"c4": {"forward": bytes, ...}, ...} plus the
+# SHA-256 of the kernel sources they were measured on.  `traffic` is null for a configuration or call that
+# was not profiled, and for every call once the kernel sources differ from the profiled ones.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+CSRC = os.path.join(ROOT, "deform_conv3d_pytorch_op_amd", "csrc")
+
+
+def csrc_sha256():
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".h", ".hip")):
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
 
 
 def measured_traffic(config, call):
     try:
         with open(TRAFFIC_FILE) as f:
-            v = json.load(f).get(config, {}).get(call)
+            table = json.load(f)
+        if table.get("_csrc_sha256") != csrc_sha256():
+            return None
+        v = table.get(config, {}).get(call)
         return float(v) if v is not None else None
     except (OSError, ValueError):
         return None
