@@ -75,6 +75,17 @@ template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G,
     const size_t packed = packed4 > packed8 ? packed4 : packed8;
     return align256((plain > packed ? plain : packed) * sizeof(T));
 }
+// Partial outputs of a forward pass that splits the input channels of a position block over several
+// workgroups: only layers of few positions do (too few blocks to fill the device), with at most
+// FWD_MAX_SPLIT parts and FWD_PARTIAL_CAP bytes.
+constexpr int FWD_MAX_SPLIT = 16;
+constexpr size_t FWD_PARTIAL_CAP = (size_t)64 << 20;
+constexpr size_t FWD_SPLIT_POSITIONS = 256 * 512;      // no split from this many positions on: they fill the device anyway
+size_t forward_partial_bound(int N, int C_out, size_t outV, size_t elem) {
+    if ((size_t)N * outV >= FWD_SPLIT_POSITIONS) return 0;
+    const size_t all = (size_t)FWD_MAX_SPLIT * N * C_out * outV * elem;
+    return align256(all < FWD_PARTIAL_CAP ? all : FWD_PARTIAL_CAP) + 256;
+}
 template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G, int cpg = 0) {
     const int M = C_out / G, Cg = C_in / G;
     int MT, mchunks, Mp, Cgp;
@@ -85,7 +96,7 @@ template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t i
     const int Mp8 = ((M + TNf - 1) / TNf + 7) / 8 * 8 * TNf;
     const size_t fwd_plain = (size_t)G * kV * (Mp > Mp8 ? Mp : Mp8) * Cgp * sizeof(T);
     const size_t fwd_quad = slab_bound((size_t)C_in, G, cpg, FQ) * forward_slab_elems<T>(kV, Mp8) * sizeof(T);
-    const size_t fwd = fwd_plain > fwd_quad ? fwd_plain : fwd_quad;
+    const size_t fwd = (fwd_plain > fwd_quad ? fwd_plain : fwd_quad) + forward_partial_bound(N, C_out, outV, sizeof(T));
     const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G, cpg) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
     // backward_weight: two channels-last copies + one partial weight per position split (at most 256 splits,
     // and never more than about 4096 workgroups: see bww_plan)
@@ -166,6 +177,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_HALO_MARGIN        voxels of halo beyond the integer tap span on each side (default 2)
 //   DCN_LDS_BUDGET_KB      LDS per 512-thread workgroup of the forward halo kernel (default 72: two per CU)
 //   DCN_FORWARD_WG=512     never use the 1024-thread forward variant; =1024 use it whenever its halo fits
+//   DCN_FORWARD_SPLIT=n    forward pass: split the input channels of a position block over at most n workgroups (0: never)
 //   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
@@ -244,6 +256,10 @@ static bool fused_tail_split() {        // DCN_FUSED_TAIL=0: the fused backward 
 }
 static int forced_slots() {             // DCN_FUSED_SLOTS=n (test hook): plan the fused backward launch as if n workgroups ran at once
     static const int v = [] { const char* e = getenv("DCN_FUSED_SLOTS"); return e && atoi(e) > 0 ? atoi(e) : 0; }();
+    return v;
+}
+static int forward_split() {            // DCN_FORWARD_SPLIT=n: the forward pass splits the input channels of a position block at most n ways
+    static const int v = [] { const char* e = getenv("DCN_FORWARD_SPLIT"); return e ? atoi(e) : 1 << 20; }();
     return v;
 }
 static bool scatter_in_lds() {
@@ -372,16 +388,34 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
     if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
     T* wt = static_cast<T*>(ws);
     const int TN = Mma<T>::TN;
-    // Small position counts with many output channels: fewer row tiles per wavefront (more output
-    // channel chunks, each sampling for itself) until there is a workgroup for every CU.
+    // Too few position blocks to give every CU a workgroup.  First the input channels of a block are
+    // split over up to FWD_MAX_SPLIT workgroups (each samples its own channels once; their partial
+    // outputs are joined by a second kernel), as far as the workspace holds the partial outputs.
+    // Then fewer row tiles per wavefront: more output-channel chunks, each sampling for itself.
+    int fsplit = 1;
+    const int mtiles_all = (P.M + TN - 1) / TN;
+    const size_t out_bytes = (size_t)P.N * P.C_out * P.outV * sizeof(T);
+    const size_t wq_bound = align256(((size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1) *
+                                     forward_slab_elems<T>(P.kV, (mtiles_all + 7) / 8 * 8 * TN) * sizeof(T));
     {
         Params Pt = P;
-        const long long tiles = plan_halo<T, ND>(Pt, 144 * 1024) ? (long long)Pt.N * Pt.tiles
-                                                                  : (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN));
-        const int mtiles = (P.M + TN - 1) / TN;
-        while (MT > 1 && tiles * P.G * P.mchunks < cu_count()) {
+        const bool tiled = plan_halo<T, ND>(Pt, 144 * 1024, 1 << 30, sizeof(T), WAVESH, false, FQ);
+        const long long tiles = tiled ? (long long)Pt.N * Pt.tiles : (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN));
+        // (eight row tiles per wavefront only pay when the grid is full anyway: measured slower than
+        // four with twice the sampling)
+        if (MT == 8 && tiles * P.G * P.mchunks < cu_count()) {
+            MT = 4;
+            P.mchunks = (mtiles_all + MT - 1) / MT;
+        }
+        if (tiled && forward_split() > 1 && (size_t)P.N * P.outV < FWD_SPLIT_POSITIONS && ws_bytes > wq_bound) {
+            const size_t room = ws_bytes - wq_bound < FWD_PARTIAL_CAP ? ws_bytes - wq_bound : FWD_PARTIAL_CAP;
+            while (fsplit * 2 <= FWD_MAX_SPLIT && fsplit * 2 <= forward_split() && tiles * P.G * P.mchunks * fsplit * 2 <= cu_count() &&
+                   (size_t)fsplit * 2 * out_bytes <= room && fsplit * 2 * FQ <= P.Cg)
+                fsplit *= 2;
+        }
+        while (MT > 1 && tiles * P.G * P.mchunks * fsplit < cu_count()) {
             MT /= 2;
-            P.mchunks = (mtiles + MT - 1) / MT;
+            P.mchunks = (mtiles_all + MT - 1) / MT;
         }
         P.Mp = P.mchunks * MT * TN;
     }
@@ -410,7 +444,21 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
         }
         const size_t slabs = (size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1;
         const size_t wq_bytes = slabs * forward_slab_elems<T>(P.kV, P.Mp) * sizeof(T);
+        if (nw == 16 || ws_bytes < align256(wq_bytes) + (size_t)fsplit * out_bytes) fsplit = 1;
         if (nw && ws_bytes >= wq_bytes) {
+            if (fsplit > 1) {
+                // channels per LDS pass such that every workgroup of a block gets the same number of passes
+                auto chunks_of_group0 = [&](int cc) {
+                    int n = 0;
+                    for (int dg = 0; dg <= (P.Cg - 1) / P.cpg; ++dg) {
+                        const int len = (P.Cg < (dg + 1) * P.cpg ? P.Cg : (dg + 1) * P.cpg) - dg * P.cpg;
+                        n += (len + cc - 1) / cc;
+                    }
+                    return n;
+                };
+                for (int cc = Ph.cchunk; cc >= FQ; cc -= FQ)
+                    if (chunks_of_group0(cc) % fsplit == 0) { Ph.cchunk = cc; break; }
+            }
             {
                 const size_t total = (size_t)P.C_in * forward_slab_elems<T>(P.kV, P.Mp);
                 const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
@@ -418,17 +466,27 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
                 if (int rc = check_launch("pack_forward_weight_kernel")) return rc;
             }
             const size_t lds = (size_t)Ph.cchunk * Ph.hstride * sizeof(T) + (size_t)Ph.hvol * 4;
-            const dim3 grid((unsigned)Ph.N * Ph.tiles * Ph.G * Ph.mchunks);
+            const dim3 grid((unsigned)Ph.N * Ph.tiles * Ph.G * Ph.mchunks * fsplit);
+            T* part = reinterpret_cast<T*>(static_cast<char*>(ws) + align256(wq_bytes));
+            T* dst = fsplit > 1 ? part : out;
+            const T* kbias = fsplit > 1 ? nullptr : bias;
+            int rc;
             if (nw == 16) {
-                if (MT == 1) return launch_halo(forward_quad_kernel<T, ND, 1, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, bias, out);
-                return launch_halo(forward_quad_kernel<T, ND, 2, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, bias, out);
+                rc = MT == 1 ? launch_halo(forward_quad_kernel<T, ND, 1, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit)
+                             : launch_halo(forward_quad_kernel<T, ND, 2, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit);
+            } else {
+                switch (MT) {
+                    case 1: rc = launch_halo(forward_quad_kernel<T, ND, 1, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    case 2: rc = launch_halo(forward_quad_kernel<T, ND, 2, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    case 4: rc = launch_halo(forward_quad_kernel<T, ND, 4, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    default: rc = launch_halo(forward_quad_kernel<T, ND, 8, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                }
             }
-            switch (MT) {
-                case 1: return launch_halo(forward_quad_kernel<T, ND, 1, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
-                case 2: return launch_halo(forward_quad_kernel<T, ND, 2, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
-                case 4: return launch_halo(forward_quad_kernel<T, ND, 4, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
-                default: return launch_halo(forward_quad_kernel<T, ND, 8, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, bias, out);
-            }
+            if (rc || fsplit == 1) return rc;
+            const size_t total = (size_t)P.N * P.C_out * P.outV;
+            const unsigned jb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+            hipLaunchKernelGGL(forward_join_partials_kernel<T>, dim3(jb), dim3(256), 0, s, part, bias, out, fsplit, total, P.C_out, P.outV);
+            return check_launch("forward_join_partials_kernel");
         }
     }
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;

@@ -76,14 +76,18 @@ __device__ inline void halo_stage_quads(const Params& P, const T* __restrict__ c
     }
 }
 
-// 1-D grid of N * tiles (3-D blocks of positions) * G * mchunks workgroups of NW wavefronts;
+// 1-D grid of N * tiles (blocks of positions) * G * mchunks * csplit workgroups of NW wavefronts;
 // dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4 with cchunk a multiple of four.
+// csplit > 1 (layers with too few position blocks to fill the device): the csplit workgroups of a
+// (block, group, output-channel chunk) share its input-channel chunks -- workgroup cz takes every
+// csplit-th -- and write their partial sums, without bias, to out + cz * N * C_out * outV;
+// forward_join_partials_kernel adds them up in a fixed order.
 // (few accumulators: four wavefronts per SIMD, i.e. at most 128 registers, also for the 512-thread
 // shape, so that two of its workgroups share a CU)
 template <typename T, int ND, int MT, int NW>
 __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, const T* __restrict__ in,
                                                            const T* __restrict__ off, const T* __restrict__ Wq,
-                                                           const T* __restrict__ bias, T* __restrict__ out) {
+                                                           const T* __restrict__ bias, T* __restrict__ out, int csplit) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, WGS = NW * 64;
     typedef T V4 __attribute__((ext_vector_type(4)));
@@ -93,7 +97,9 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     // workgroups of one tile are neighbours in an XCD-contiguous order
-    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+    const unsigned wgs = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int cz = wgs % (unsigned)csplit;
+    const unsigned wg = wgs / (unsigned)csplit;
     const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
     const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
 
@@ -129,10 +135,12 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     const unsigned w_tg = (unsigned)mtiles * KL * TN * FQ;        // one tap group further
 
     const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
+    int chunk_no = 0;
     for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
         const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
         const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
         for (int cc0 = cb; cc0 < ce; cc0 += P.cchunk) {
+            if ((chunk_no++) % csplit != cz) continue;                     // another workgroup's chunk (uniform)
             const int nch = min(P.cchunk, ce - cc0);
             const int ngrp = (nch + FQ - 1) / FQ;
             const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
@@ -289,6 +297,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     }
 
     if (!valid) return;
+    T* dst = out + (size_t)cz * P.N * P.C_out * P.outV;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -297,9 +306,21 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
             if (m < P.M) {
                 T v = acc[mt][r];
                 if (bias) v += bias[g * P.M + m];
-                out[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+                dst[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
             }
         }
+}
+
+// out = bias + the sum of `parts` partial outputs of forward_quad_kernel, added in the order of the
+// parts (the result does not depend on which workgroup finished first).
+template <typename T>
+__global__ void forward_join_partials_kernel(const T* __restrict__ part, const T* __restrict__ bias, T* __restrict__ out,
+                                             int parts, size_t total, int C_out, unsigned outV) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        T v = part[i];
+        for (int s = 1; s < parts; ++s) v += part[(size_t)s * total + i];
+        out[i] = bias ? v + bias[(i / outV) % (size_t)C_out] : v;
+    }
 }
 
 }  // namespace dcn
