@@ -11,6 +11,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <utility>
 
 namespace {
@@ -187,6 +188,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_CSPLIT=n           fused backward kernel: every item split over n workgroups
 //   DCN_FUSED_SLOTS=n      fused backward kernel: plan the launch as if n workgroups ran at once (test hook)
 //   DCN_FUSED_FIXED=0      fused backward kernel: runtime plane stride even where the compile-time one fits
+//   DCN_FUSED_PAIR=0       fused backward kernel, float32: one channel per 64-bit LDS cell instead of two 32-bit halves
 static size_t env_kb(const char* name, int dflt) {
     const char* e = getenv(name);
     const int v = e ? atoi(e) : dflt;
@@ -261,6 +263,10 @@ static int forced_slots() {             // DCN_FUSED_SLOTS=n (test hook): plan t
 static int forward_split() {            // DCN_FORWARD_SPLIT=n: the forward pass splits the input channels of a position block at most n ways
     static const int v = [] { const char* e = getenv("DCN_FORWARD_SPLIT"); return e ? atoi(e) : 1 << 20; }();
     return v;
+}
+static bool fused_pair() {              // DCN_FUSED_PAIR=0: float32 LDS cells of the fused backward kernel hold one channel each (64-bit)
+    static const int v = [] { const char* e = getenv("DCN_FUSED_PAIR"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
 }
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
@@ -512,6 +518,19 @@ int absmax(const T* w, size_t n, float* out, hipStream_t s) {
     hipLaunchKernelGGL(absmax_kernel<T>, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, n, out);
     return check_launch("absmax_kernel");
 }
+// out[0] = max |w|, out[1] = largest norm over the output channels of a group of an (input channel, tap) column
+template <typename T>
+int weight_bounds(const Params& P, const T* w, float* out, hipStream_t s) {
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(1), dim3(64), 0, s, out, (size_t)2);
+    if (int rc = check_launch("fill_zero_kernel")) return rc;
+    const size_t n = (size_t)P.C_out * P.Cg * P.kV, cols = (size_t)P.Cg * P.kV;
+    const unsigned blocks = (unsigned)((n + 1023) / 1024 > 128 ? 128 : (n + 1023) / 1024);
+    hipLaunchKernelGGL(absmax_kernel<T>, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, n, out);
+    if (int rc = check_launch("absmax_kernel")) return rc;
+    if (P.G > 65535) return fail(DCN_E_ARGUMENT, "more than 65535 convolution groups");
+    hipLaunchKernelGGL(colnorm_max_kernel<T>, dim3((unsigned)((cols + 63) / 64), (unsigned)P.G), dim3(512), 0, s, w, P.M, cols, out + 1);
+    return check_launch("colnorm_max_kernel");
+}
 
 template <typename T, int ND>
 int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* off, const T* gout, T* gin,
@@ -540,24 +559,33 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     // Eight wavefronts per workgroup; four (half the positions, in the block shape with the smallest
     // halo) where only that fits, e.g. under stride 2.
     constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
-    for (int nw = fused_first_waves(); nw >= 4 && scatter_in_lds() && fused_coord(); nw /= 2) {
+    // (attempts: eight wavefronts on the default block, eight on the block shape with the smallest
+    // halo, four on the block shape with the smallest halo)
+    for (int attempt = fused_first_waves() == 8 ? 0 : 2; attempt < 3 && scatter_in_lds() && fused_coord(); ++attempt) {
+        const int nw = attempt < 2 ? 8 : 4;
+        const bool smallest = attempt > 0;
         Params Ph = P;
-        if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, 8 + sizeof(T), nw, nw == 4)) continue;
+        // float32: two channels per LDS cell as 32-bit fixed point while the terms one cell can receive
+        // (positions of the block x taps) leave at least 17 bits below the largest possible term
+        const bool pair = sizeof(T) == 4 && fused_pair() && (long long)nw * TN * P.kV <= (1 << 14);
+        const size_t chb = (pair ? 4 : 8) + sizeof(T);      // LDS bytes per channel and halo voxel: cell + input value
+        if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, chb, nw, smallest)) continue;
         const size_t tables = (size_t)Ph.hvol * 4;      // halo table
-        const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * (8 + sizeof(T)) + tables <= scatter_budget();
+        const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * chb + tables <= scatter_budget();
         if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
-        if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) < 4) continue;
+        if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) < 4) continue;
         // Channels per chunk: 8 where that takes fewer MFMA passes per channel (a pass holds TN / CCH
-        // taps: the 9 taps of a 3x3 kernel are 2 float passes per 4 channels or 3 per 8) and the
-        // planes of 8 channels fit, which the small halos of 2-D layers allow.
+        // taps: the 9 taps of a 3x3 kernel are 2 float passes per 4 channels or 3 per 8; the 27 of a
+        // 3x3x3 kernel 4 or 7) and the planes of 8 channels fit: the small halos of 2-D layers, and
+        // 3-D ones with paired cells.
         const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;
         auto passes = [&](int c) { const int tp = Mma<T>::TN / c; return (P.kV + tp - 1) / tp; };
-        const bool eight = ND == 2 && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
-                           (scatter_budget() - tables) / ((size_t)Ph.hstride * (8 + sizeof(T))) >= 8;
+        const bool eight = (ND == 2 || pair) && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
+                           (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 8;
         const int cch = eight ? 8 : 4;
         Ph.cchunk = cch;
         if (fixed && !eight) Ph.hstride = FUSED_HS;
-        const size_t lds = (size_t)cch * Ph.hstride * (8 + sizeof(T)) + tables;
+        const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
         {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
             const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in, cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
@@ -565,24 +593,30 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt);
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
-        if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
+        if (int rc = weight_bounds<T>(P, w, wmax, s)) return rc;
         // grad_output operand held in registers when its reduction steps fit: 8 per tap slot of a pass
         // (M <= 64 float, 128 double with 4-channel chunks)
         const int slot_regs = (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
         const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= Mma<T>::NACC / slot_regs * 8;
         using Kern = void (*)(Params, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
         Kern kern = nullptr;
-#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true>
-#define DCN_FUSED(BREG_, HS_, NW_) DCN_FUSED_C(4, BREG_, HS_, NW_)
-        if constexpr (ND == 2) {
-            if (eight) kern = breg ? DCN_FUSED_C(8, true, 0, 8) : DCN_FUSED_C(8, false, 0, 8);
-        }
-        if (!kern) {
-            if (nw == 8) kern = fixed && breg ? DCN_FUSED(true, FUSED_HS, 8) : fixed ? DCN_FUSED(false, FUSED_HS, 8) : DCN_FUSED(false, 0, 8);
-            else kern = fixed && breg ? DCN_FUSED(true, FUSED_HS, 4) : fixed ? DCN_FUSED(false, FUSED_HS, 4) : DCN_FUSED(false, 0, 4);
-        }
-#undef DCN_FUSED
+#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>
+        auto pick = [&](auto pair_tag) {
+            constexpr bool PR = decltype(pair_tag)::value;
+            if (eight) {
+                if constexpr (ND == 2 || PR) kern = breg ? DCN_FUSED_C(8, true, 0, 8, PR) : DCN_FUSED_C(8, false, 0, 8, PR);
+            } else if (nw == 8)
+                kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 8, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 8, PR) : DCN_FUSED_C(4, false, 0, 8, PR);
+            else
+                kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 4, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 4, PR) : DCN_FUSED_C(4, false, 0, 4, PR);
+        };
+        if constexpr (sizeof(T) == 4) {
+            if (pair) pick(std::true_type{});
+            else pick(std::false_type{});
+        } else
+            pick(std::false_type{});
 #undef DCN_FUSED_C
+        if (!kern) continue;
         if (lds > 48 * 1024)
             if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return rc;
         // Work items are (tile, deformable group) pairs, each a run of nchunks channel chunks.  `slots`

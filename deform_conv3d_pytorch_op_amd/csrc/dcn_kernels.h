@@ -806,6 +806,22 @@ template <> struct LdsCell<float> {
     __device__ static inline float value(type c, double inv_scale) {
         return (float)((double)((long long)(c << 16) >> 16) * inv_scale);      // sign-extended low 48 bits
     }
+    // Two channels in one cell: signed 32-bit integers a (low half) and b (high half) are added as
+    // the single 64-bit number b * 2^32 + a, i.e. with b lowered by one where a is negative, so
+    // that any number of terms sums exactly in both halves as long as each half's sum fits 32
+    // bits (the caller scales the terms accordingly).
+    __device__ static inline void add2(type* p, double w, double g0_scaled, double g1_scaled) {
+        const int a = (int)__double_as_longlong(__builtin_fma(w, g0_scaled, MAGIC));      // low 32 bits = the integer mod 2^32
+        const int b = (int)__double_as_longlong(__builtin_fma(w, g1_scaled, MAGIC)) + (a >> 31);
+        const type v = ((type)(unsigned)b << 32) | (type)(unsigned)a;
+        (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __device__ static inline void value2(type c, double inv_scale, float& v0, float& v1) {
+        const int a = (int)(unsigned)c;
+        const int b = (int)(unsigned)(c >> 32) - (a >> 31);        // undo the borrow of a negative low half
+        v0 = (float)((double)a * inv_scale);
+        v1 = (float)((double)b * inv_scale);
+    }
 };
 template <> struct LdsCell<double> {
     typedef double type;
@@ -834,6 +850,33 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
         __syncthreads();
     }
     if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned*>(out), redu[0]);
+}
+
+// max over the weight's (input channel, tap) columns of the Euclidean norm over the output channels
+// of one convolution group, NaN if any element is NaN: |grad column| <= that norm times the norm of
+// grad_output over the output channels at the position (Cauchy-Schwarz).  W is [G*M][Cg][kV];
+// grid (ceil(Cg*kV / 64), G); joined like absmax_kernel.  `out` must hold 0 beforehand.
+template <typename T>
+__global__ __launch_bounds__(512) void colnorm_max_kernel(const T* __restrict__ w, int M, size_t cols, float* __restrict__ out) {
+    // workgroup = 64 neighbouring columns of one group (blockIdx.y) x 8 slices of its rows
+    __shared__ float part[8][64];
+    const int cx = threadIdx.x & 63, sl = threadIdx.x >> 6;
+    const size_t col = (size_t)blockIdx.x * 64 + cx;
+    float ss = 0.f;
+    if (col < cols) {
+        const T* p = w + (size_t)blockIdx.y * M * cols + col;
+#pragma unroll 8
+        for (int r = sl; r < M; r += 8) { const float v = (float)p[(size_t)r * cols]; ss += v * v; }
+    }
+    part[sl][cx] = ss;
+    __syncthreads();
+    if (sl == 0) {
+#pragma unroll
+        for (int k = 1; k < 8; ++k) ss += part[k][cx];
+        unsigned m = __float_as_uint(fabsf(sqrtf(ss)));       // NaN keeps the largest pattern
+        for (int sh = 1; sh < 64; sh <<= 1) m = max(m, (unsigned)__shfl_xor((int)m, sh));
+        if (cx == 0) atomicMax(reinterpret_cast<unsigned*>(out), m);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -867,7 +910,12 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
 // of a channel becomes an immediate offset of the LDS instructions instead of address arithmetic.
 // PACKW: the weights come in the per-chunk lane order of pack_weight_kernel instead of
 // [g][tap][m][channel].
-template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false>
+// PAIR (float only): the cells hold two channels each as 32-bit fixed point (LdsCell<float>::add2):
+// half the LDS atomics and two thirds of the LDS bytes per channel.  The terms are scaled such
+// that (positions of the block x taps) of the largest possible one -- all that a cell can receive
+// -- still fit 31 bits; the host allows it only while that leaves enough bits below that term.
+// wmax[1] then holds the largest column norm of the weight (colnorm_max_kernel).
+template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false>
 __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
@@ -882,10 +930,12 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     constexpr int RPS = (MM::row(1, 0) - MM::row(0, 0) == 1) ? 4 : CCH / 4;   // registers that share a tap
     constexpr int NS = NACC / RPS;                      // tap slots per lane and pass
     static_assert(TN % CCH == 0 && CCH % 4 == 0 && NACC % RPS == 0, "unsupported channel chunk");
+    static_assert(!PAIR || (sizeof(T) == 4 && RPS % 2 == 0), "paired cells are a float32 layout");
+    constexpr int CPL = PAIR ? CCH / 2 : CCH;           // cell planes
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int hs = HS ? HS : P.hstride;
-    Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CCH][hstride]
-    T* sIn = reinterpret_cast<T*>(sG + (size_t)CCH * hs);                               // [hstride][CCH] if COORD: channels of a voxel side by side
+    Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CPL][hstride]
+    T* sIn = reinterpret_cast<T*>(sG + (size_t)CPL * hs);                               // [hstride][CCH] if COORD: channels of a voxel side by side
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
     constexpr int WGS = NW * 64;                        // threads per workgroup
     __shared__ float sRed[NW];
@@ -952,7 +1002,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         const unsigned b_byte = b_off * (unsigned)sizeof(T);
         const unsigned b_byte_last = (klast * KL + q < P.M ? b_off : pos) * (unsigned)sizeof(T);
         T b_reg[BREG ? NS * AB : 1];
-        float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share)
+        float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share); PAIR: of the squares
         if constexpr (BREG) {
             // held unmasked (rows past M meet zero weight rows, columns outside the volume are never
             // used): a masked load becomes a conditional one, issued alone with a full wait behind it
@@ -968,7 +1018,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 gk += k < kl ? gstep * sizeof(T) : (size_t)0;
             }
 #pragma unroll
-            for (int k = 0; k < NS * AB; ++k) sabs += (valid && (k < kl || (k == kl && kl * KL + q < P.M))) ? fabsf((float)b_reg[k]) : 0.f;
+            for (int k = 0; k < NS * AB; ++k) {
+                const float bk = (float)b_reg[k];
+                sabs += (valid && (k < kl || (k == kl && kl * KL + q < P.M))) ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
+            }
         } else {
             // unconditional loads, eight in flight, masked when they are summed (a masked load
             // becomes a conditional one that is waited for on its own)
@@ -983,7 +1036,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                 for (int k = 0; k < AB; ++k) {
                     const int kk_ = k0 + k;
-                    sabs += (valid && (kk_ < klast || (kk_ == klast && klast * KL + q < P.M))) ? fabsf((float)bv[k]) : 0.f;
+                    const float bk = (float)bv[k];
+                    sabs += (valid && (kk_ < klast || (kk_ == klast && klast * KL + q < P.M))) ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
                 }
             }
         }
@@ -1002,19 +1056,26 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
         for (int w8 = 0; w8 < NW; ++w8) smaxb = max(smaxb, __float_as_uint(sRed[w8]));
         int ex = 0;
-        const float bound = 8.f * wmax[0] * __uint_as_float(smaxb);
+        // paired cells: |term| <= largest column norm of W x largest norm of grad_output over the
+        // output channels (0.1 % slack for the rounding of those two and of the MFMA sums)
+        const float bound = PAIR ? 1.001f * wmax[1] * sqrtf(__uint_as_float(smaxb)) : 8.f * wmax[0] * __uint_as_float(smaxb);
         // the LDS cells need a finite bound; without one this workgroup scatters through the far path
         // (float cells need the exponent; and with either cell type a corner that carries weight zero
         // would receive 0 * inf = NaN where the reference adds nothing)
         const bool cells_ok = bound < 3.0e38f;                        // false for NaN
         if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
-        const double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
+        double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
+        if constexpr (PAIR) {
+            // all the terms a cell can receive, each at the bound, stay below 2^31
+            scale = bound > 0.f && bound < 3.0e38f ? 2147483648.0 * 0.99 / ((double)(NW * TN) * P.kV * (double)bound) : 1.0;
+            inv_scale = 1.0 / scale;
+        }
 
         for (int cc0 = rb; cc0 < re; cc0 += CCH) {
             if ((chunk_no++) % cs != cz) continue;          // another workgroup's chunk (uniform)
             const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
-            for (int c = 0; c < nch; ++c)
+            for (int c = 0; c < (PAIR ? (nch + 1) / 2 : nch); ++c)
                 for (int v = threadIdx.x; v < P.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
             if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
@@ -1297,12 +1358,22 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     }
                     if (near) {
                         Cell* cp = sG + base;
+                        if constexpr (PAIR) {
 #pragma unroll
-                        for (int rr = 0; rr < RPS; ++rr) {
-                            const double gs = LdsCell<T>::pre(gv[rr], scale);
-                            const int cl = MM::row(ts * RPS + rr, q) % CCH;
+                            for (int rr = 0; rr < RPS; rr += 2) {          // consecutive registers hold consecutive channels
+                                const double g0 = LdsCell<T>::pre(gv[rr], scale), g1 = LdsCell<T>::pre(gv[rr + 1], scale);
+                                const int pl = (MM::row(ts * RPS + rr, q) % CCH) / 2;
 #pragma unroll
-                            for (int i = 0; i < NC; ++i) LdsCell<T>::add(cp + coff[i] + cl * hs, (double)cw[i], gs);
+                                for (int i = 0; i < NC; ++i) LdsCell<T>::add2(cp + coff[i] + pl * hs, (double)cw[i], g0, g1);
+                            }
+                        } else {
+#pragma unroll
+                            for (int rr = 0; rr < RPS; ++rr) {
+                                const double gs = LdsCell<T>::pre(gv[rr], scale);
+                                const int cl = MM::row(ts * RPS + rr, q) % CCH;
+#pragma unroll
+                                for (int i = 0; i < NC; ++i) LdsCell<T>::add(cp + coff[i] + cl * hs, (double)cw[i], gs);
+                            }
                         }
                     }
                     if constexpr (COORD && ND == 3) {
@@ -1399,10 +1470,23 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             for (int v = threadIdx.x; v < P.hvol; v += WGS) {
                 const unsigned gv = sTab[v];
                 if (gv == ~0u) continue;            // halo cell outside the volume: never touched
-                for (int c = 0; c < nch; ++c) {
-                    const Cell cell = sG[c * hs + v];
-                    if (cell != (Cell)0)
-                        atomic_add(gin + ((size_t)n * P.C_in + cc0 + c) * P.inV + gv, (T)LdsCell<T>::value(cell, inv_scale));
+                if constexpr (PAIR) {
+                    for (int c = 0; c < nch; c += 2) {
+                        const Cell cell = sG[(c / 2) * hs + v];
+                        if (cell != (Cell)0) {
+                            float v0, v1;
+                            LdsCell<float>::value2(cell, inv_scale, v0, v1);
+                            T* gp = gin + ((size_t)n * P.C_in + cc0 + c) * P.inV + gv;
+                            if (v0 != 0.f) atomic_add(gp, (T)v0);
+                            if (c + 1 < nch && v1 != 0.f) atomic_add(gp + P.inV, (T)v1);
+                        }
+                    }
+                } else {
+                    for (int c = 0; c < nch; ++c) {
+                        const Cell cell = sG[c * hs + v];
+                        if (cell != (Cell)0)
+                            atomic_add(gin + ((size_t)n * P.C_in + cc0 + c) * P.inV + gv, (T)LdsCell<T>::value(cell, inv_scale));
+                    }
                 }
             }
         }
