@@ -41,14 +41,14 @@ def load():
     tail = [_c_vp, _c_sz, _c_vp]            # workspace, workspace_bytes, stream
     for nd in (2, 3):
         geom = [_c_int] * N_GEOM[nd]
-        for suf in ("f32", "f64"):
+        for suf in ("f32", "f64", "bf16", "f16"):
             f = getattr(L, "dcn%dd_forward_%s" % (nd, suf))
             f.restype, f.argtypes = _c_int, [_c_vp] * 5 + geom + tail
             f = getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))
             f.restype, f.argtypes = _c_int, [_c_vp] * 6 + geom + tail
             f = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
             f.restype, f.argtypes = _c_int, [_c_vp] * 4 + geom + tail
-            if nd == 3:
+            if nd == 3 and suf in ("f32", "f64"):
                 f = getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)
                 f.restype, f.argtypes = _c_int, [_c_vp] * 6 + geom + tail + [ctypes.c_uint]
     L.dcn3d_forward_noalloc_f32.restype = _c_int
@@ -66,7 +66,8 @@ def check(rc):
 
 EXPORTS = ["dcn_version", "dcn_arch", "dcn_last_error", "dcn_workspace_bytes", "dcn_workspace_bytes_for"] + [
     "dcn%dd_%s_%s" % (nd, op, suf)
-    for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight") for suf in ("f32", "f64")] + [
+    for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight")
+    for suf in ("f32", "f64", "bf16", "f16")] + [
     "dcn3d_backward_input_offset_flags_f32", "dcn3d_backward_input_offset_flags_f64",
     "dcn3d_forward_noalloc_f32"]
 NOALLOC_SCRATCH_BYTES = 8 << 20

@@ -826,6 +826,100 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     return check_launch("reduce_weight_partials_kernel");
 }
 
+// ---------------------------------------------------------------------------------------------
+// Mixed precision: tensors stored as bfloat16 / binary16, arithmetic in float32.  The tensors are
+// widened into float copies at the front of the workspace, the float32 kernels run on them with the
+// rest of the workspace, and the results are rounded once.
+struct Carver {
+    char* p;
+    size_t left;
+    float* take(size_t n) {
+        const size_t b = align256(n * sizeof(float));
+        if (!p || b > left) return nullptr;
+        float* r = reinterpret_cast<float*>(p);
+        p += b;
+        left -= b;
+        return r;
+    }
+};
+template <typename S> int widen(const S* src, float* dst, size_t n, hipStream_t s) {
+    const unsigned blocks = (unsigned)((n + 1023) / 1024 > 8192 ? 8192 : (n + 1023) / 1024);
+    hipLaunchKernelGGL(widen_kernel<S>, dim3(blocks ? blocks : 1), dim3(256), 0, s, src, dst, n);
+    return check_launch("widen_kernel");
+}
+template <typename S> int narrow(const float* src, S* dst, size_t n, hipStream_t s) {
+    const unsigned blocks = (unsigned)((n + 1023) / 1024 > 8192 ? 8192 : (n + 1023) / 1024);
+    hipLaunchKernelGGL(narrow_kernel<S>, dim3(blocks ? blocks : 1), dim3(256), 0, s, src, dst, n);
+    return check_launch("narrow_kernel");
+}
+struct Sizes16 { size_t in, w, off, out; };
+Sizes16 sizes16(const Params& P, int nd) {
+    return Sizes16{(size_t)P.N * P.C_in * P.inV, (size_t)P.C_out * P.Cg * P.kV, (size_t)P.N * P.DG * P.kV * nd * P.outV,
+                   (size_t)P.N * P.C_out * P.outV};
+}
+// float copies of every tensor any of the three calls touches (nd = 3 bounds the offsets of either operator)
+size_t copies16_bytes(int N, int C_in, int C_out, size_t inV, size_t outV, int kV, int G, int cpg) {
+    const size_t in = (size_t)N * C_in * inV, w = (size_t)C_out * (C_in / G) * kV, off = (size_t)N * (C_in / cpg) * kV * 3 * outV,
+                 out = (size_t)N * C_out * outV;
+    return 2 * align256(in * 4) + 2 * align256(w * 4) + 2 * align256(off * 4) + align256(out * 4) + align256((size_t)C_out * 4);
+}
+
+template <typename S, int ND>
+int forward16(const Geometry& g, const S* in, const S* w, const S* off, const S* bias, S* out, void* ws, size_t ws_bytes,
+              hipStream_t s) {
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    if (!in || !w || !off || !out) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    if (int rc = device_info(nullptr)) return rc;
+    const Sizes16 z = sizes16(P, ND);
+    Carver c{static_cast<char*>(ws), ws ? ws_bytes : 0};
+    float *fin = c.take(z.in), *fw = c.take(z.w), *foff = c.take(z.off), *fout = c.take(z.out), *fb = bias ? c.take(P.C_out) : nullptr;
+    if (!fin || !fw || !foff || !fout || (bias && !fb)) return fail(DCN_E_WORKSPACE, "workspace too small");
+    if (int rc = widen(in, fin, z.in, s)) return rc;
+    if (int rc = widen(w, fw, z.w, s)) return rc;
+    if (int rc = widen(off, foff, z.off, s)) return rc;
+    if (bias) if (int rc = widen(bias, fb, (size_t)P.C_out, s)) return rc;
+    if (int rc = forward<float, ND>(g, fin, fw, foff, fb, fout, c.p, c.left, s)) return rc;
+    return narrow(fout, out, z.out, s);
+}
+template <typename S, int ND>
+int backward_input_offset16(const Geometry& g, const S* in, const S* w, const S* off, const S* gout, S* gin, S* goff, void* ws,
+                            size_t ws_bytes, hipStream_t s) {
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    if (int rc = device_info(nullptr)) return rc;
+    const Sizes16 z = sizes16(P, ND);
+    Carver c{static_cast<char*>(ws), ws ? ws_bytes : 0};
+    float *fin = c.take(z.in), *fw = c.take(z.w), *foff = c.take(z.off), *fgout = c.take(z.out), *fgin = c.take(z.in), *fgoff = c.take(z.off);
+    if (!fin || !fw || !foff || !fgout || !fgin || !fgoff) return fail(DCN_E_WORKSPACE, "workspace too small");
+    if (int rc = widen(in, fin, z.in, s)) return rc;
+    if (int rc = widen(w, fw, z.w, s)) return rc;
+    if (int rc = widen(off, foff, z.off, s)) return rc;
+    if (int rc = widen(gout, fgout, z.out, s)) return rc;
+    if (int rc = widen(gin, fgin, z.in, s)) return rc;            // grad_input is accumulated into
+    if (int rc = backward_input_offset<float, ND>(g, fin, fw, foff, fgout, fgin, fgoff, c.p, c.left, s)) return rc;
+    if (int rc = narrow(fgin, gin, z.in, s)) return rc;
+    return narrow(fgoff, goff, z.off, s);
+}
+template <typename S, int ND>
+int backward_weight16(const Geometry& g, const S* in, const S* off, const S* gout, S* gw, void* ws, size_t ws_bytes, hipStream_t s) {
+    Params P;
+    if (int rc = validate(g, P)) return rc;
+    if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    if (int rc = device_info(nullptr)) return rc;
+    const Sizes16 z = sizes16(P, ND);
+    Carver c{static_cast<char*>(ws), ws ? ws_bytes : 0};
+    float *fin = c.take(z.in), *foff = c.take(z.off), *fgout = c.take(z.out), *fgw = c.take(z.w);
+    if (!fin || !foff || !fgout || !fgw) return fail(DCN_E_WORKSPACE, "workspace too small");
+    if (int rc = widen(in, fin, z.in, s)) return rc;
+    if (int rc = widen(off, foff, z.off, s)) return rc;
+    if (int rc = widen(gout, fgout, z.out, s)) return rc;
+    if (int rc = widen(gw, fgw, z.w, s)) return rc;               // grad_weight is accumulated into
+    if (int rc = backward_weight<float, ND>(g, fin, foff, fgout, fgw, c.p, c.left, s)) return rc;
+    return narrow(fgw, gw, z.w, s);
+}
+
 Geometry geo3(int batch, int input_c, int output_c, int input_l, int input_h, int input_w, int output_l,
               int output_h, int output_w, int kernel_l, int kernel_h, int kernel_w, int pad_l, int pad_h,
               int pad_w, int stride_l, int stride_h, int stride_w, int dilation_l, int dilation_h,
@@ -888,7 +982,7 @@ const char* dcn_last_error(void) { return g_err.c_str(); }
 size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
                            size_t output_volume, int kernel_volume, int group) {
     if (group <= 0 || batch <= 0 || input_c <= 0 || output_c <= 0 || kernel_volume <= 0 || input_volume == 0 ||
-        output_volume == 0)
+        output_volume == 0 || elem_size == 2)      // 16-bit storage: dcn_workspace_bytes_for
         return 0;
     return elem_size == 8
                ? workspace_need<double>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group)
@@ -901,6 +995,9 @@ size_t dcn_workspace_bytes_for(int elem_size, int batch, int input_c, int output
         output_volume == 0 || channel_per_deformable_group <= 0 || input_c % channel_per_deformable_group)
         return 0;
     const int cpg = channel_per_deformable_group;
+    if (elem_size == 2)     // bfloat16 / binary16 storage: float copies of the tensors + the float32 workspace
+        return copies16_bytes(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg) +
+               workspace_need<float>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg);
     return elem_size == 8
                ? workspace_need<double>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg)
                : workspace_need<float>(batch, input_c, output_c, input_volume, output_volume, kernel_volume, group, cpg);
@@ -975,5 +1072,48 @@ int dcn3d_forward_noalloc_f32(const float* input, const float* weight, const flo
 
 DEFINE_OPS(f32, float)
 DEFINE_OPS(f64, double)
+
+#define DEFINE_OPS16(SUF, S)                                                                                        \
+    int dcn3d_forward_##SUF(const void* input, const void* weight, const void* offset, const void* bias, void* output, \
+                            DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {                \
+        return forward16<S, 3>(geo3(G3_ARGS), (const S*)input, (const S*)weight, (const S*)offset, (const S*)bias,  \
+                               (S*)output, workspace, workspace_bytes, static_cast<hipStream_t>(stream));           \
+    }                                                                                                               \
+    int dcn3d_backward_input_offset_##SUF(const void* input, const void* weight, const void* offset,                \
+                                          const void* grad_output, void* grad_input, void* grad_offset,             \
+                                          DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {  \
+        return backward_input_offset16<S, 3>(geo3(G3_ARGS), (const S*)input, (const S*)weight, (const S*)offset,    \
+                                             (const S*)grad_output, (S*)grad_input, (S*)grad_offset, workspace,     \
+                                             workspace_bytes, static_cast<hipStream_t>(stream));                    \
+    }                                                                                                               \
+    int dcn3d_backward_weight_##SUF(const void* input, const void* offset, const void* grad_output,                 \
+                                    void* grad_weight, DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes,     \
+                                    void* stream) {                                                                 \
+        return backward_weight16<S, 3>(geo3(G3_ARGS), (const S*)input, (const S*)offset, (const S*)grad_output,     \
+                                       (S*)grad_weight, workspace, workspace_bytes,                                 \
+                                       static_cast<hipStream_t>(stream));                                           \
+    }                                                                                                               \
+    int dcn2d_forward_##SUF(const void* input, const void* weight, const void* offset, const void* bias, void* output, \
+                            DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {                \
+        return forward16<S, 2>(geo2(G2_ARGS), (const S*)input, (const S*)weight, (const S*)offset, (const S*)bias,  \
+                               (S*)output, workspace, workspace_bytes, static_cast<hipStream_t>(stream));           \
+    }                                                                                                               \
+    int dcn2d_backward_input_offset_##SUF(const void* input, const void* weight, const void* offset,                \
+                                          const void* grad_output, void* grad_input, void* grad_offset,             \
+                                          DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes, void* stream) {  \
+        return backward_input_offset16<S, 2>(geo2(G2_ARGS), (const S*)input, (const S*)weight, (const S*)offset,    \
+                                             (const S*)grad_output, (S*)grad_input, (S*)grad_offset, workspace,     \
+                                             workspace_bytes, static_cast<hipStream_t>(stream));                    \
+    }                                                                                                               \
+    int dcn2d_backward_weight_##SUF(const void* input, const void* offset, const void* grad_output,                 \
+                                    void* grad_weight, DCN2D_GEOMETRY, void* workspace, size_t workspace_bytes,     \
+                                    void* stream) {                                                                 \
+        return backward_weight16<S, 2>(geo2(G2_ARGS), (const S*)input, (const S*)offset, (const S*)grad_output,     \
+                                       (S*)grad_weight, workspace, workspace_bytes,                                 \
+                                       static_cast<hipStream_t>(stream));                                           \
+    }
+
+DEFINE_OPS16(bf16, Bf16)
+DEFINE_OPS16(f16, Fp16)
 
 }  // extern "C"

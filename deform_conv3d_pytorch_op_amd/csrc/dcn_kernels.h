@@ -544,6 +544,33 @@ __global__ void add_from_channels_last_kernel(const T* __restrict__ src, T* __re
     }
 }
 
+// 16-bit storage formats of the mixed-precision entry points: the tensors are widened to float
+// (exactly) before the float32 kernels run and the results are rounded once, to nearest even.
+struct Bf16 {       // bfloat16: the upper half of a float
+    unsigned short bits;
+    __device__ static inline float widen(Bf16 v) { return __uint_as_float((unsigned)v.bits << 16); }
+    __device__ static inline Bf16 narrow(float f) {
+        const unsigned u = __float_as_uint(f);
+        Bf16 r;
+        if ((u & 0x7fffffffu) > 0x7f800000u) r.bits = (unsigned short)((u >> 16) | 0x40u);      // NaN stays NaN
+        else r.bits = (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);                  // Inf and overflow to Inf included
+        return r;
+    }
+};
+struct Fp16 {       // IEEE binary16
+    _Float16 v;
+    __device__ static inline float widen(Fp16 x) { return (float)x.v; }
+    __device__ static inline Fp16 narrow(float f) { Fp16 r; r.v = (_Float16)f; return r; }
+};
+template <typename S>
+__global__ void widen_kernel(const S* __restrict__ src, float* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::widen(src[i]);
+}
+template <typename S>
+__global__ void narrow_kernel(const float* __restrict__ src, S* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::narrow(src[i]);
+}
+
 template <typename T>
 __global__ void fill_zero_kernel(T* __restrict__ p, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;

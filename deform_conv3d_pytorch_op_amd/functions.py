@@ -24,7 +24,7 @@ from torch.autograd.function import once_differentiable
 
 from . import _lib
 
-_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.bfloat16: "bf16", torch.float16: "f16"}
 
 
 def _check(cond, msg):
@@ -86,7 +86,7 @@ def _device_check(*tensors):
     t0 = tensors[0]
     _check(t0.is_cuda, "deformable convolution runs on the GPU only: tensors must be on a HIP device "
                        "(there is no CPU path in this package)")
-    _check(t0.dtype in _SUFFIX, "dtype must be float32 or float64")
+    _check(t0.dtype in _SUFFIX, "dtype must be float32, float64, bfloat16 or float16")
     for t in tensors[1:]:
         if t is None:
             continue
@@ -192,6 +192,7 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
             args = (inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
                     grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, main.cuda_stream)
             if nd == 3 and oob_zero:        # the reference's 2-D kernels have no out-of-range term
+                _check(suf in ("f32", "f64"), "oob_offset_grad='zero' is available in float32 and float64 only")
                 _lib.check(getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)(*args, _lib.FLAG_OOB_OFFSET_GRAD_ZERO))
             else:
                 _lib.check(getattr(L, "dcn%dd_backward_input_offset_%s" % (nd, suf))(*args))

@@ -61,7 +61,8 @@ int dcn_version(void);              /* ABI version, currently 1 */
 const char *dcn_arch(void);         /* the code-object target the kernels were built for: "gfx950" */
 const char *dcn_last_error(void);   /* message of the last failing call on this thread ("" if none) */
 
-/* Scratch bytes any of the three calls below needs for this layer (elem_size 4 = f32, 8 = f64;
+/* Scratch bytes any of the three calls below needs for this layer (elem_size 4 = f32, 8 = f64; the
+ * 16-bit formats, elem_size 2, are served by dcn_workspace_bytes_for only and get 0 here;
  * input_volume = input_l * input_h * input_w, output_volume likewise, kernel_volume =
  * kernel_l * kernel_h * kernel_w).  The workspace holds a re-laid-out copy of the weight and, for
  * the backward calls, channels-last copies of the input batch, its gradient and grad_output. */
@@ -161,6 +162,52 @@ int dcn2d_backward_weight_f32(const float *input, const float *offset, const flo
 int dcn2d_backward_weight_f64(const double *input, const double *offset, const double *grad_output,
                               double *grad_weight, DCN2D_GEOMETRY, void *workspace,
                               size_t workspace_bytes, void *stream);
+
+/* ---- 16-bit storage, float32 arithmetic ------------------------------------------------------
+ * No counterpart in the reference, which instantiates float only
+ * (deform3d/lib/deform_conv3d_cuda_kernel.cu:162-172).  Every tensor (input, weight, offset, bias,
+ * grad_output and the results) is stored as bfloat16 (_bf16) or IEEE binary16 (_f16); the values are
+ * widened exactly, all products and sums are the float32 kernels', and each result element is
+ * rounded once, to nearest even.  Same argument meaning and accumulate / overwrite contract as
+ * the _f32 calls (grad_input and grad_weight: rounded sum of their previous content and the
+ * gradient).  The workspace must come from dcn_workspace_bytes_for(2, ...): it also holds float
+ * copies of the tensors.  Offsets in 16 bits limit the sampling positions to that format's grid
+ * (bfloat16: 1/128 voxel between 1 and 2, coarser above). */
+int dcn3d_forward_bf16(const void *input, const void *weight, const void *offset, const void *bias,
+                       void *output, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn3d_backward_input_offset_bf16(const void *input, const void *weight, const void *offset,
+                                     const void *grad_output, void *grad_input, void *grad_offset,
+                                     DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn3d_backward_weight_bf16(const void *input, const void *offset, const void *grad_output,
+                               void *grad_weight, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes,
+                               void *stream);
+
+int dcn2d_forward_bf16(const void *input, const void *weight, const void *offset, const void *bias,
+                       void *output, DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn2d_backward_input_offset_bf16(const void *input, const void *weight, const void *offset,
+                                     const void *grad_output, void *grad_input, void *grad_offset,
+                                     DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn2d_backward_weight_bf16(const void *input, const void *offset, const void *grad_output,
+                               void *grad_weight, DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes,
+                               void *stream);
+
+int dcn3d_forward_f16(const void *input, const void *weight, const void *offset, const void *bias,
+                       void *output, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn3d_backward_input_offset_f16(const void *input, const void *weight, const void *offset,
+                                     const void *grad_output, void *grad_input, void *grad_offset,
+                                     DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn3d_backward_weight_f16(const void *input, const void *offset, const void *grad_output,
+                               void *grad_weight, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes,
+                               void *stream);
+
+int dcn2d_forward_f16(const void *input, const void *weight, const void *offset, const void *bias,
+                       void *output, DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn2d_backward_input_offset_f16(const void *input, const void *weight, const void *offset,
+                                     const void *grad_output, void *grad_input, void *grad_offset,
+                                     DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
+int dcn2d_backward_weight_f16(const void *input, const void *offset, const void *grad_output,
+                               void *grad_weight, DCN2D_GEOMETRY, void *workspace, size_t workspace_bytes,
+                               void *stream);
 
 #ifdef __cplusplus
 }

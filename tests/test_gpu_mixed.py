@@ -1,0 +1,76 @@
+"""16-bit storage entry points (dcn*_bf16, dcn*_f16) through the package's Functions: every tensor is
+stored as bfloat16 / binary16, the arithmetic is the float32 kernels' and each result is rounded
+once.  Oracle mode: the CPU oracle in float64 on the same 16-bit-rounded inputs.  A result then
+differs from the oracle by the float32 kernels' error plus one rounding to the storage format,
+half an ulp of the element: 2^-9 of its magnitude for bfloat16, 2^-12 for binary16.  Tolerances,
+relative to the tensor's largest magnitude: bfloat16 5e-3, binary16 1e-3 forward / 2e-3 gradients.
+The reference has no such mode (deform3d/lib/deform_conv3d_cuda_kernel.cu:162-172 instantiates float only).
+"""
+import pytest
+import torch
+
+from oracle import dcn_oracle as orc
+from tests.cases import SMALL_CASES, make_case
+from tests.test_gpu_parity import rel_err, run_gpu
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: dict(fwd=5e-3, grad=5e-3), torch.float16: dict(fwd=1e-3, grad=2e-3)}
+CASES = ["2d_basic", "2d_c3_like", "2d_wide_m", "2d_chunk8_ragged", "3d_basic", "3d_mixed", "3d_c4_like", "3d_c5_like",
+         "3d_short_length"]
+MEDIUM = {   # several position blocks, more than one channel chunk
+    "3d_medium": (3, 2, 24, 40, (6, 20, 18), 3, 1, 1, 1, 12, 1, 2.0),
+    "2d_medium": (2, 2, 48, 64, (30, 34), 3, 1, 1, 1, 16, 2, 2.0),
+}
+
+
+def _compare(c, dtype, tag):
+    got = run_gpu(c)
+    for g in got:
+        assert g is None or g.dtype == dtype
+    wide = {k: (v.double() if torch.is_tensor(v) else v) for k, v in c.items()}
+    cfg = (c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+    want = (orc.forward(wide["x"], wide["off"], wide["w"], wide["b"], *cfg),) + tuple(
+        orc.backward(wide["x"], wide["off"], wide["w"], wide["gout"], wide["b"], *cfg))
+    for name, g, w in zip(("output", "grad_input", "grad_offset", "grad_weight", "grad_bias"), got, want):
+        if w is None:
+            continue
+        tol = TOL[dtype]["fwd" if name == "output" else "grad"]
+        e = rel_err(g.float(), w)
+        assert e <= tol, "%s %s: relative error %.3e > %.1e" % (tag, name, e, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("name", CASES)
+def test_16bit_storage_small_cases_match_oracle(name, dtype):
+    print("16-bit case", name, dtype, flush=True)
+    _compare(make_case(*SMALL_CASES[name], dtype=dtype, seed=7), dtype, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("name", sorted(MEDIUM))
+def test_16bit_storage_medium_cases_match_oracle(name, dtype):
+    print("16-bit case", name, dtype, flush=True)
+    _compare(make_case(*MEDIUM[name], dtype=dtype, seed=8), dtype, name)
+
+
+def test_16bit_results_are_the_float32_results_rounded_once():
+    """The bfloat16 output equals the float32 kernel's output on the widened inputs, rounded to bfloat16."""
+    import deform_conv3d_pytorch_op_amd as dcn
+    c = make_case(*SMALL_CASES["3d_c4_like"], dtype=torch.bfloat16, seed=9)
+    dev = torch.device("cuda:0")
+    x, off, w, b = (c[k].to(dev) for k in ("x", "off", "w", "b"))
+    cfg = (c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+    out16 = dcn.ConvOffset3dFunction.apply(x, off, w, b, *cfg)
+    out32 = dcn.ConvOffset3dFunction.apply(x.float(), off.float(), w.float(), b.float(), *cfg)
+    assert torch.equal(out16, out32.to(torch.bfloat16))
+
+
+def test_oob_zero_switch_is_float_only():
+    import deform_conv3d_pytorch_op_amd as dcn
+    c = make_case(*SMALL_CASES["3d_basic"], dtype=torch.float16, seed=1)
+    dev = torch.device("cuda:0")
+    x, off, w = (c[k].to(dev).requires_grad_(True) for k in ("x", "off", "w"))
+    out = dcn.ConvOffset3dFunction.apply(x, off, w, None, c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"], False, "zero")
+    with pytest.raises(RuntimeError, match="float32 and float64 only"):
+        out.backward(c["gout"].to(dev))
