@@ -59,7 +59,7 @@ constexpr int TAP_PAD = 8;      // zero tap slabs behind the last group: an MFMA
 // `cch` channels) for `slabs` slabs.
 template <typename T> size_t packed_weight_elems(int M, int kV, size_t slabs, int cch) {
     const int KL = Mma<T>::KL, TP = Mma<T>::TN / cch;
-    return slabs * ((kV + TP - 1) / TP) * (size_t)(((M + KL - 1) / KL + 7) / 8 * 8) * 64;
+    return slabs * ((kV + TP - 1) / TP) * (size_t)(((M + KL - 1) / KL + 15) / 16 * 16) * 64;
 }
 // Upper bound of chunk_slot<cch>(cpg, Cg, c) + 1 over the channels: the slabs a per-chunk weight
 // layout occupies.  cpg = 0: the channels per deformable group are not known (the first workspace
@@ -586,18 +586,22 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         Ph.cchunk = cch;
         if (fixed && !eight) Ph.hstride = FUSED_HS;
         const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
+        // grad_output operand held in registers when its reduction steps fit: 32 per pass
+        // (M <= 64 float, 128 double with 4-channel chunks)
+        const int ksteps = (P.M + Mma<T>::KL - 1) / Mma<T>::KL;
+        const bool wide = eight && pair && ksteps <= 32;                                         // the kernel's WIDE
+        const int slot_regs = wide ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
+        const bool breg = ksteps <= Mma<T>::NACC / slot_regs * (wide ? 16 : 8);
         {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
             const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in, cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
-            if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), dim3(blocks), dim3(256), 0, s, P, w, wt);
+            // (wide: row order that leaves the eight channels of a tap in one lane)
+            if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), dim3(blocks), dim3(256), 0, s, P, w, wt);
+            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), dim3(blocks), dim3(256), 0, s, P, w, wt);
             else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt);
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
         if (int rc = weight_bounds<T>(P, w, wmax, s)) return rc;
-        // grad_output operand held in registers when its reduction steps fit: 8 per tap slot of a pass
-        // (M <= 64 float, 128 double with 4-channel chunks)
-        const int slot_regs = (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
-        const bool breg = (P.M + Mma<T>::KL - 1) / Mma<T>::KL <= Mma<T>::NACC / slot_regs * 8;
         using Kern = void (*)(Params, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
         Kern kern = nullptr;
 #define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>

@@ -47,12 +47,15 @@ __global__ void relayout_weight_kernel(Params P, const T* __restrict__ W, T* __r
 template <int CCH>
 __host__ __device__ inline int chunk_slot(int cpg, int Cg, int c0) { return c0 / CCH + c0 / cpg + c0 / Cg; }
 
-template <typename T, int CCH>
+// WIDE (float, CCH = 8): row j of a pass holds (tap, channel) = (2 * (j / 16) + (j / 4) % 2,
+// 4 * ((j / 8) % 2) + j % 4) instead of (j / CCH, j % CCH): the MFMA then leaves all eight channels
+// of a tap in one lane (fused_row_tap / fused_row_channel).
+template <typename T, int CCH, bool WIDE = false>
 __global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, TP = TN / CCH;
     const int npass = (P.kV + TP - 1) / TP;
-    const int kst = ((P.M + KL - 1) / KL + 7) / 8 * 8;          // operand batches are 8 reduction steps
+    const int kst = ((P.M + KL - 1) / KL + 15) / 16 * 16;       // operand batches are 8 or 16 reduction steps
     const size_t per_chunk = (size_t)npass * kst * 64;
     const size_t total = (size_t)P.C_in * per_chunk;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
@@ -63,7 +66,8 @@ __global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restr
         const size_t r = i % per_chunk;
         const int lane = (int)(r % 64), k = (int)((r / 64) % kst), pass = (int)(r / 64 / kst);
         const int q = lane / TN, j = lane % TN;
-        const int m = k * KL + q, tap = pass * TP + j / CCH, c = c0 + j % CCH, g = c0 / P.Cg;
+        const int jt = WIDE ? 2 * (j / 16) + (j / 4) % 2 : j / CCH, jc = WIDE ? 4 * ((j / 8) % 2) + j % 4 : j % CCH;
+        const int m = k * KL + q, tap = pass * TP + jt, c = c0 + jc, g = c0 / P.Cg;
         T v = 0;
         if (m < P.M && tap < P.kV && c < seg_e) v = W[(((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap];
         Wp[(size_t)chunk_slot<CCH>(P.cpg, P.Cg, c0) * per_chunk + r] = v;
@@ -954,8 +958,16 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
     constexpr int TP = TN / CCH;                        // taps per MFMA pass
-    constexpr int RPS = (MM::row(1, 0) - MM::row(0, 0) == 1) ? 4 : CCH / 4;   // registers that share a tap
+    // WIDE (paired cells, 8-channel chunks): the weight rows are ordered such that a lane receives
+    // all eight channels of a tap -- lane group q the taps q and 2 + q of a pass -- instead of four
+    // channels of each of four taps, with the other four in the other lane group: the geometry of a
+    // (tap, position) is then worked out once per eight channels, not once per lane group.
+    constexpr bool WIDE = PAIR && CCH == 8 && BREG;      // (with the grad_output operand in registers: measured slower without)
+    constexpr int RPS = WIDE ? 8 : (MM::row(1, 0) - MM::row(0, 0) == 1) ? 4 : CCH / 4;   // registers that share a tap
     constexpr int NS = NACC / RPS;                      // tap slots per lane and pass
+    // (tap of the pass, channel of the chunk) behind accumulator register r of lane group qq
+    auto row_tap = [](int r, int qq) { return WIDE ? 2 * (r / 8) + qq : MM::row(r, qq) / CCH; };
+    auto row_ch = [](int r, int qq) { return WIDE ? r % 8 : MM::row(r, qq) % CCH; };
     static_assert(TN % CCH == 0 && CCH % 4 == 0 && NACC % RPS == 0, "unsupported channel chunk");
     static_assert(!PAIR || (sizeof(T) == 4 && RPS % 2 == 0), "paired cells are a float32 layout");
     constexpr int CPL = PAIR ? CCH / 2 : CCH;           // cell planes
@@ -1013,7 +1025,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
         // wave-uniform base (scalar registers) + 32-bit lane offset of the B operand grad_output[m][pos]
-        constexpr int AB = 8;                       // reduction steps per operand batch
+        constexpr int AB = WIDE ? 16 : 8;           // reduction steps per operand batch (NS * AB = 32 ride on a pass)
         const T* gbase = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV;
         const unsigned b_off = (unsigned)q * P.outV + pos;
         const size_t gstep = (size_t)KL * P.outV;
@@ -1115,7 +1127,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             constexpr int MPR = AB / RPS;                              // MFMAs per accumulator register walked
             const int ksteps = (P.M + KL - 1) / KL;
             const size_t wstep = PACKW ? (size_t)64 : (size_t)KL * P.Cgp;
-            const size_t wpass = PACKW ? (size_t)((ksteps + 7) / 8 * 8) * 64 : (size_t)TP * P.Mp * P.Cgp;   // weights of one pass
+            const size_t wpass = PACKW ? (size_t)((ksteps + 15) / 16 * 16) * 64 : (size_t)TP * P.Mp * P.Cgp;   // weights of one pass
             const T* wchunk = PACKW ? Wt + (size_t)chunk_slot<CCH>(P.cpg, P.Cg, cc0) * ((P.kV + TP - 1) / TP) * wpass
                                     : Wt + ((size_t)g * P.kV * P.Mp) * P.Cgp + (cc0 - g * P.Cg);      // uniform; lanes add a_off
             // (k0 passes through an empty asm: what is derived from it is then computed where it is
@@ -1201,12 +1213,12 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             constexpr int STEP = TP / NS;
             static_assert(TP % NS == 0, "taps of consecutive slots are evenly spaced");
             int kq[ND];
-            decode_tap<ND>(P, MM::row(0, q) / CCH, kq);
+            decode_tap<ND>(P, row_tap(0, q), kq);
             auto load_slot_offsets = [&](int tap_u, int ts) {         // tap_u: uniform tap of lane group 0 in slot ts
                 T* o_nx = o_buf[ts & 1];
                 T* kd_nx = kd_buf[ts & 1];
                 const int tu = min(tap_u, P.kV - 1);
-                const int dq = MM::row(ts * RPS, q) / CCH - MM::row(ts * RPS, 0) / CCH;
+                const int dq = row_tap(ts * RPS, q) - row_tap(ts * RPS, 0);
                 const int dqc = tu + dq < P.kV ? dq : 0;
                 const unsigned lo = (unsigned)dqc * ND * P.outV + pos;
                 const T* ob = off_dg + (size_t)tu * ND * P.outV;
@@ -1226,7 +1238,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     kq[0] += carry;
                 }
             };
-            load_slot_offsets(MM::row(0, 0) / CCH, 0);
+            load_slot_offsets(row_tap(0, 0), 0);
             // grad_offset of a finished tap slot, held back until the loads of the next slot have been
             // issued: vector memory operations complete in order, so a load issued behind these
             // stores / atomics could only be waited for together with them
@@ -1266,8 +1278,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
                     // slots past the last tap (only in the last pass, which feeds no further MFMAs)
-                    if (tap0 + MM::row(ts * RPS, 0) / CCH >= P.kV) continue;
-                    const int tap = tap0 + MM::row(ts * RPS, q) / CCH;
+                    if (tap0 + row_tap(ts * RPS, 0) >= P.kV) continue;
+                    const int tap = tap0 + row_tap(ts * RPS, q);
                     T a_cu[AB], b_cu[AB];
                     const T* ofs = o_buf[ts & 1];
                     const T* kdf = kd_buf[ts & 1];
@@ -1275,8 +1287,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     // this slot's MFMA operands arrive while its geometry is set up; the offsets of the
                     // next tap slot travel while this one is worked on
                     if (do_mma) load_batch(a_cu, b_cu, wnext, ts * AB);
-                    if (ts + 1 < NS) load_slot_offsets(tap0 + MM::row((ts + 1) * RPS, 0) / CCH, ts + 1);
-                    else load_slot_offsets(tap0 + TP + MM::row(0, 0) / CCH, 0);
+                    if (ts + 1 < NS) load_slot_offsets(tap0 + row_tap((ts + 1) * RPS, 0), ts + 1);
+                    else load_slot_offsets(tap0 + TP + row_tap(0, 0), 0);
                     __builtin_amdgcn_sched_barrier(0);
                     if constexpr (COORD) write_goff();
                     __builtin_amdgcn_sched_barrier(0);
@@ -1330,42 +1342,50 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                     for (int rr = 0; rr < RPS; ++rr) {
                         gv[rr] = d[ts * RPS + rr];
-                        if constexpr (!PACKW) gv[rr] = (MM::row(ts * RPS + rr, q) % CCH) < nch ? gv[rr] : (T)0;
+                        if constexpr (!PACKW) gv[rr] = row_ch(ts * RPS + rr, q) < nch ? gv[rr] : (T)0;
                     }
-                    // corner values of the input: one wide LDS read per corner for all of this lane's
-                    // channels, issued by every lane, ahead of the MFMAs that cover their latency
-                    T vv[NC][RPS];
-                    if constexpr (COORD) {
-                        const T* ip = sIn + (size_t)base * CCH;
+                    // Corner values of the input: one wide LDS read per corner for four of this lane's
+                    // channels, issued by every lane, ahead of the MFMAs that cover their latency.
+                    // d(sample)/d(coordinate) is linear in the corner values: it is applied once to
+                    // the corner values weighted by gcol and summed over the lane's channels.  Every
+                    // lane does this, outside any branch (a lane without a near sample works on cell
+                    // 0 and drops the result): corner reads still pending at a branch that skips
+                    // their use would make the compiler wait for the whole LDS queue, adds included,
+                    // before the registers are written again.  Eight channels per slot go in two
+                    // rounds of four (reads, half of the slot's MFMAs, sums) to bound the registers.
+                    constexpr int RH = RPS > 4 ? RPS / 4 : 1, RW = RPS / RH;
+                    T v[NC];
 #pragma unroll
-                        for (int i = 0; i < NC; ++i)
+                    for (int h = 0; h < RH; ++h) {
+                        T vv[NC][RW];
+                        if constexpr (COORD) {
+                            const T* ip = sIn + (size_t)base * CCH;
 #pragma unroll
-                            for (int rr = 0; rr < RPS; ++rr) vv[i][rr] = ip[coff[i] * CCH + MM::row(ts * RPS + rr, q) % CCH];
-                    }
-                    // the next pass's MFMAs of this slot, in uniform control flow
-                    if (do_mma) {
+                            for (int i = 0; i < NC; ++i)
 #pragma unroll
-                        for (int k = 0; k < AB; ++k)
-                            d_next = MM::mma(a_cu[k], BREG ? b_reg[ts * AB + k] : b_cu[k], d_next);
+                                for (int rr = 0; rr < RW; ++rr) vv[i][rr] = ip[coff[i] * CCH + row_ch(ts * RPS + h * RW + rr, q)];
+                        }
+                        // the next pass's MFMAs of this slot, in uniform control flow
+                        if (do_mma) {
+#pragma unroll
+                            for (int k = h * (AB / RH); k < (h + 1) * (AB / RH); ++k)
+                                d_next = MM::mma(a_cu[k], BREG ? b_reg[ts * AB + k] : b_cu[k], d_next);
+                        }
+                        if constexpr (COORD) {
+#pragma unroll
+                            for (int i = 0; i < NC; ++i) {
+                                T acc_ = h == 0 ? gv[0] * vv[i][0] : v[i] + gv[h * RW] * vv[i][0];
+#pragma unroll
+                                for (int rr = 1; rr < RW; ++rr) acc_ += gv[h * RW + rr] * vv[i][rr];
+                                v[i] = acc_;
+                            }
+                        }
+                        if (h + 1 < RH) __builtin_amdgcn_sched_barrier(0);
                     }
                     T ga[ND];
 #pragma unroll
                     for (int a = 0; a < ND; ++a) ga[a] = 0;
                     if constexpr (COORD) {
-                        // d(sample)/d(coordinate) is linear in the corner values: it is applied once to
-                        // the corner values weighted by gcol and summed over the lane's channels.  Every
-                        // lane does this, outside any branch (a lane without a near sample works on cell
-                        // 0 and drops the result): corner reads still pending at a branch that skips
-                        // their use would make the compiler wait for the whole LDS queue, adds included,
-                        // before the registers are written again.
-                        T v[NC];
-#pragma unroll
-                        for (int i = 0; i < NC; ++i) {
-                            T acc_ = gv[0] * vv[i][0];
-#pragma unroll
-                            for (int rr = 1; rr < RPS; ++rr) acc_ += gv[rr] * vv[i][rr];
-                            v[i] = acc_;
-                        }
                         if constexpr (ND == 3) {
                             const T fl = f[0], gl = (T)1 - fl, fh = f[1], gh = (T)1 - fh, fw = f[2], gw = (T)1 - fw;
                             const T c00 = v[0] * gw + v[1] * fw, c01 = v[2] * gw + v[3] * fw;
@@ -1389,7 +1409,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                             for (int rr = 0; rr < RPS; rr += 2) {          // consecutive registers hold consecutive channels
                                 const double g0 = LdsCell<T>::pre(gv[rr], scale), g1 = LdsCell<T>::pre(gv[rr + 1], scale);
-                                const int pl = (MM::row(ts * RPS + rr, q) % CCH) / 2;
+                                const int pl = row_ch(ts * RPS + rr, q) / 2;
 #pragma unroll
                                 for (int i = 0; i < NC; ++i) LdsCell<T>::add2(cp + coff[i] + pl * hs, (double)cw[i], g0, g1);
                             }
@@ -1397,7 +1417,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                             for (int rr = 0; rr < RPS; ++rr) {
                                 const double gs = LdsCell<T>::pre(gv[rr], scale);
-                                const int cl = MM::row(ts * RPS + rr, q) % CCH;
+                                const int cl = row_ch(ts * RPS + rr, q);
 #pragma unroll
                                 for (int i = 0; i < NC; ++i) LdsCell<T>::add(cp + coff[i] + cl * hs, (double)cw[i], gs);
                             }
@@ -1444,7 +1464,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         }
 #pragma unroll
                         for (int rr = 0; rr < RPS; ++rr) {
-                            const int cl = MM::row(ts * RPS + rr, q) % CCH;
+                            const int cl = row_ch(ts * RPS + rr, q);
                             if (far && cl < nch) {
                                 const T g1 = gv[rr];
                                 const size_t chan = ((size_t)n * P.C_in + cc0 + cl + kz) * P.inV;
