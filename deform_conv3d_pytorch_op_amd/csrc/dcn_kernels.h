@@ -239,34 +239,7 @@ __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsign
     }
 }
 
-// Stage `nch` channel planes of the halo.  Halo voxels outside the volume are never read by a
-// sample; they are staged from voxel 0 so that every load is unconditional.
-template <typename T, int WGS = WGH>
-__device__ inline void halo_stage(const Params& P, const T* __restrict__ chan0, int nch,
-                                  const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
-    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGS * 4) {
-        unsigned g[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int v = v0 + WGS * k;
-            const unsigned t = v < P.hvol ? sTab[v] : ~0u;
-            g[k] = t == ~0u ? 0u : t;
-        }
-        for (int c = 0; c < nch; ++c) {
-            const T* ch = chan0 + (size_t)c * P.inV;
-            T val[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) val[k] = ch[g[k]];              // four loads in flight
-            // unconditional stores (past the last voxel: into the plane's last padding cell, which is
-            // never read), so that the loads above are not folded into conditional blocks and waited
-            // for one by one
-#pragma unroll
-            for (int k = 0; k < 4; ++k) sIn[c * P.hstride + (v0 + WGS * k < P.hvol ? v0 + WGS * k : P.hstride - 1)] = val[k];
-        }
-    }
-}
-
-// The same for a channel-interleaved halo [halo voxel][CCH]: the CCH channel values of a voxel sit
+// Stage `nch` channels of the halo channel-interleaved, [halo voxel][CCH]: the CCH channel values of a voxel sit
 // next to each other, so one wide LDS read fetches a corner of all of them (missing channels of a
 // short last chunk and halo voxels outside the volume are stored as zero).
 template <typename T, int CCH, int WGS>
@@ -282,226 +255,6 @@ __device__ inline void halo_stage_interleaved(const Params& P, const T* __restri
 #pragma unroll
         for (int c = 0; c < CCH; ++c) sIn[(size_t)v * CCH + c] = (c < nch && t != ~0u) ? val[c] : (T)0;
     }
-}
-
-// LDS indices of the corners of an inside sample; false if any corner lies outside the halo
-template <typename T, int ND>
-__device__ inline bool halo_corners(const Params& P, const int hb[ND], const TapGeo<T, ND>& t, unsigned lidx[1 << ND]) {
-    bool in_halo = true;
-    int l[ND], h[ND];
-#pragma unroll
-    for (int a = 0; a < ND; ++a) {
-        l[a] = t.lo[a] - hb[a];
-        h[a] = t.hi[a] - hb[a];
-        in_halo = in_halo && l[a] >= 0 && h[a] < P.hext[slot<ND>(a)];
-    }
-    if constexpr (ND == 3) {
-        const int e1 = P.hext[1], e2 = P.hext[2];
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-            lidx[c] = in_halo ? (unsigned)((((c & 4) ? h[0] : l[0]) * e1 + ((c & 2) ? h[1] : l[1])) * e2 + ((c & 1) ? h[2] : l[2])) : 0u;
-    } else {
-        const int e2 = P.hext[2];
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-            lidx[c] = in_halo ? (unsigned)(((c & 2) ? h[0] : l[0]) * e2 + ((c & 1) ? h[1] : l[1])) : 0u;
-    }
-    return in_halo;
-}
-
-// The same indices at fewer instructions (used by the fused backward kernel; the forward kernel
-// keeps the form above, with which it compiles to faster code).  The low corner's index takes two 24-bit multiply-adds (halo
-// coordinates and extents are far below 2^24; 32-bit integer multiplies run at a quarter of the
-// rate) and the other corners are that index plus the strides of the axes whose high corner has
-// not collapsed onto the low one.
-template <typename T, int ND>
-__device__ inline bool halo_corners_strided(const Params& P, const int hb[ND], const TapGeo<T, ND>& t, unsigned lidx[1 << ND]) {
-    bool in_halo = true;
-    int l[ND], d[ND];
-#pragma unroll
-    for (int a = 0; a < ND; ++a) {
-        l[a] = t.lo[a] - hb[a];
-        d[a] = t.hi[a] - t.lo[a];                   // 0 or 1
-        in_halo = in_halo && l[a] >= 0 && l[a] + d[a] < P.hext[slot<ND>(a)];
-    }
-    if constexpr (ND == 3) {
-        const int e1 = P.hext[1], e2 = P.hext[2], e12 = e1 * e2;
-        const int base = __mul24(__mul24(l[0], e1) + l[1], e2) + l[2];
-        const unsigned b = in_halo ? (unsigned)base : 0u;
-        const unsigned s0 = (in_halo && d[0]) ? (unsigned)e12 : 0u, s1 = (in_halo && d[1]) ? (unsigned)e2 : 0u;
-        const unsigned s2 = (in_halo && d[2]) ? 1u : 0u;
-        lidx[0] = b;           lidx[1] = b + s2;           lidx[2] = b + s1;           lidx[3] = b + s1 + s2;
-        lidx[4] = b + s0;      lidx[5] = b + s0 + s2;      lidx[6] = b + s0 + s1;      lidx[7] = b + s0 + s1 + s2;
-    } else {
-        const int e2 = P.hext[2];
-        const int base = __mul24(l[0], e2) + l[1];
-        const unsigned b = in_halo ? (unsigned)base : 0u;
-        const unsigned s0 = (in_halo && d[0]) ? (unsigned)e2 : 0u, s1 = (in_halo && d[1]) ? 1u : 0u;
-        lidx[0] = b; lidx[1] = b + s1; lidx[2] = b + s0; lidx[3] = b + s0 + s1;
-    }
-    return in_halo;
-}
-
-// Forward with the input halo in LDS.  Same contraction and lane roles as forward_kernel; the
-// sampled value of lane (j, q) is the MFMA B operand B[k = q][col = j].
-// 1-D grid of N * tiles (3-D blocks of positions) * G * mchunks, NW wavefronts per workgroup
-// (16 when the accumulators are few enough for 128 registers: the larger block shares each staged
-// halo between twice the positions); dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4.
-template <typename T, int ND, int MT, int NW>
-__global__ __launch_bounds__(NW * 64) void forward_halo_kernel(Params P, const T* __restrict__ in,
-                                                           const T* __restrict__ off, const T* __restrict__ Wt,
-                                                           const T* __restrict__ bias, T* __restrict__ out) {
-    using MM = Mma<T>;
-    constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sIn = reinterpret_cast<T*>(smem_raw);                                            // [cchunk][hstride]
-    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)P.cchunk * P.hstride);   // [hvol]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int j = lane % TN, q = lane / TN;
-    // 1-D grid of N * tiles * G * mchunks workgroups; those of one tile are neighbours
-    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
-    const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
-    const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
-
-    TileGeo<ND> tg;
-    tile_decode<ND>(P, wg / (unsigned)(P.G * P.mchunks), tg);
-    const int n = tg.n;
-    int o[ND], ib[ND];
-    unsigned pos;
-    const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
-#pragma unroll
-    for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
-    halo_table<ND, NW * 64>(P, tg, sTab);          // visible after the first barrier below
-
-    typename MM::Acc acc[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_zero<T>();
-
-    const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
-    for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
-        const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
-        const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
-        for (int cc0 = cb; cc0 < ce; cc0 += P.cchunk) {
-            const int nch = min(P.cchunk, ce - cc0);
-            const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
-            __syncthreads();                                               // readers of the previous chunk are done
-            halo_stage<T, NW * 64>(P, chan0, nch, sTab, sIn);
-            __syncthreads();
-            const int nsteps = (nch + KL - 1) / KL;
-            T onext[ND];
-            load_offsets<T, ND>(P, off_dg, pos, onext);                    // offsets of tap 0
-
-            int kk[ND];                                                    // tap coordinates, counted up with the tap (no divisions)
-#pragma unroll
-            for (int a = 0; a < ND; ++a) kk[a] = 0;
-            for (int tap = 0; tap < P.kV; ++tap) {
-                int kd[ND];
-#pragma unroll
-                for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
-#pragma unroll
-                for (int a = ND - 1; a >= 0; --a) {                        // next tap: increment with carry, fastest axis last
-                    if (++kk[a] < P.k[slot<ND>(a)] || a == 0) break;
-                    kk[a] = 0;
-                }
-                T ocur[ND];
-#pragma unroll
-                for (int a = 0; a < ND; ++a) ocur[a] = onext[a];
-                // the next tap's offsets travel while this tap is computed
-                if (tap + 1 < P.kV) load_offsets<T, ND>(P, off_dg + (size_t)(tap + 1) * ND * P.outV, pos, onext);
-                TapGeo<T, ND> t;
-                tap_setup_noidx<T, ND>(P, ocur, ib, kd, t);
-                const bool live = valid && t.inside;
-                // (a wave whose samples are all outside still multiplies its zero column rows: with a
-                // non-finite weight the reference's GEMM turns them into NaN, and so does this)
-                unsigned lidx[NC];
-                const bool in_halo = halo_corners_strided<T, ND>(P, tg.hb, t, lidx);
-                const bool near = live && in_halo;                         // sampled from LDS
-                const bool far = live && !in_halo;                         // sampled from global memory
-#pragma unroll
-                for (int c = 0; c < NC; ++c) lidx[c] += (unsigned)q * P.hstride;   // 0 + plane of this lane when !in_halo
-                const T* wrow = Wt + (((size_t)g * P.kV + tap) * P.Cgp + (cc0 - cg0) + q) * P.Mp +
-                                (size_t)mchunk * MT * TN + j;
-                // branch-free main loop: every lane reads LDS at a legal index and the value is
-                // masked afterwards; the weights of the next step are fetched one step ahead
-                if constexpr (MT <= 2 && NW == 16) {
-                    // few accumulators, four wavefronts per SIMD: the step's own weights are requested at
-                    // its top and a scheduling barrier keeps the loads there (the LDS reads, the
-                    // interpolation and the other wavefronts cover their latency); the compiler otherwise
-                    // moves one of them between the two MFMAs, where it is waited for at once
-                    const T* plane = sIn;
-                    const T* wr = wrow;
-                    for (int s = 0; s < nsteps; ++s) {
-                        T a_cur[MT];
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) a_cur[mt] = wr[mt * TN];
-                        wr += (size_t)KL * P.Mp;
-                        __builtin_amdgcn_sched_barrier(0);
-                        const T v = sample<T, ND>(plane, lidx, t.f);
-                        const T b = (near && s * KL + q < nch) ? v : (T)0;
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a_cur[mt], b, acc[mt]);
-                        plane += KL * P.hstride;
-                    }
-                } else {
-                    const T* plane = sIn;
-                    const T* wr = wrow;
-                    T a_next[MT];
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) a_next[mt] = wr[mt * TN];
-#pragma unroll 2
-                    for (int s = 0; s < nsteps; ++s) {
-                        T a_cur[MT];
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) a_cur[mt] = a_next[mt];
-                        wr += (size_t)KL * P.Mp;                           // rows past the chunk stay inside the padded weight
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) a_next[mt] = wr[mt * TN];
-                        // (few accumulators: here too the loads are kept above the step's arithmetic,
-                        // and pinned at its end they are first waited for there)
-                        if constexpr (MT <= 2) __builtin_amdgcn_sched_barrier(0);
-                        const T v = sample<T, ND>(plane, lidx, t.f);
-                        const T b = (near && s * KL + q < nch) ? v : (T)0;
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a_cur[mt], b, acc[mt]);
-                        if constexpr (MT <= 2) {
-#pragma unroll
-                            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(a_next[mt]));
-                        }
-                        plane += KL * P.hstride;
-                    }
-                }
-                if (__any(far)) {                  // rare: some sample of this wave reaches past the halo
-                    tap_corner_idx<T, ND>(P, t);
-                    unsigned voff[NC];
-#pragma unroll
-                    for (int c = 0; c < NC; ++c) voff[c] = t.idx[c] + (unsigned)q * P.inV;
-                    const T* chan = chan0;
-                    const T* wr = wrow;
-                    for (int s = 0; s < nsteps; ++s) {
-                        T b = 0;
-                        if (far && s * KL + q < nch) b = sample<T, ND>(chan, voff, t.f);
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wr[mt * TN], b, acc[mt]);
-                        chan += (size_t)KL * P.inV;
-                        wr += (size_t)KL * P.Mp;
-                    }
-                }
-            }
-        }
-    }
-
-    if (!valid) return;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int r = 0; r < MM::NACC; ++r) {
-            const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
-            if (m < P.M) {
-                T v = acc[mt][r];
-                if (bias) v += bias[g * P.M + m];
-                out[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
-            }
-        }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -915,7 +668,7 @@ __global__ __launch_bounds__(512) void colnorm_max_kernel(const T* __restrict__ 
 // deform3d kernel.cu:229-296 / deform2d_double kernel.cu:201-238, fed by the grad-column GEMM of
 // deform3d/lib/deform_conv3d_cuda.cpp:213-220).
 //
-// Same halo tiling as forward_halo_kernel, but the LDS planes hold the partial grad-input of CCH
+// Same halo tiling as forward_quad_kernel, but the LDS planes hold the partial grad-input of CCH
 // channels over the halo of the workgroup's position block (cells: see LdsCell).  The rows of
 // one MFMA tile are (tap, channel) pairs -- TP = TN / CCH taps of the CCH channels -- so a pass
 // of ceil(M / KL) MFMAs yields the grad-column values gcol[c][tap][pos] of TP taps at once with

@@ -59,6 +59,11 @@ SMALL_CASES = {
     "3d_k1_stride3": (3, 2, 5, 7, (5, 7, 6), 1, 3, 0, 1, 5, 1, 2.0),         # a single tap, odd channel counts, stride > kernel
     "3d_dilation3": (3, 1, 4, 4, (8, 8, 8), 3, 1, 3, 3, 2, 1, 2.5),          # dilation-blind output 12^3: many taps out of range
     "3d_short_length": (3, 1, 4, 4, (2, 8, 8), (1, 3, 3), 1, (0, 1, 1), 1, 4, 1, 4.0),  # D < H: out-of-range branch vs length extent
+    "3d_chunk8_ragged": (3, 1, 20, 40, (5, 9, 10), 3, 1, 1, 1, 10, 1, 2.0),     # 10-channel segments: chunks of 8 + 2, 20 reduction steps (not a multiple of 16)
+    "3d_chunk8_two_blocks": (3, 2, 16, 24, (6, 10, 18), 3, 1, 1, 1, 16, 1, 1.5),   # several position blocks per axis, 8-channel chunks, 12 reduction steps
+    "3d_k5": (3, 1, 8, 6, (6, 7, 7), 5, 1, 2, 1, 8, 1, 1.5),                  # 125 taps: too many terms per LDS cell for the paired float cells
+    "2d_k7": (2, 1, 8, 10, (12, 11), 7, 1, 3, 1, 8, 1, 2.0),                   # 49 taps
+    "3d_m72_chunk8": (3, 1, 16, 72, (4, 8, 9), 3, 1, 1, 1, 8, 1, 1.5),        # 36 reduction steps: the grad_output operand does not fit the registers
 }
 
 
