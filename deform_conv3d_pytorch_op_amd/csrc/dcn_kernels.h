@@ -594,9 +594,12 @@ template <> struct LdsCell<float> {
     // the single 64-bit number b * 2^32 + a, i.e. with b lowered by one where a is negative, so
     // that any number of terms sums exactly in both halves as long as each half's sum fits 32
     // bits (the caller scales the terms accordingly).
-    __device__ static inline void add2(type* p, double w, double g0_scaled, double g1_scaled) {
-        const int a = (int)__double_as_longlong(__builtin_fma(w, g0_scaled, MAGIC));      // low 32 bits = the integer mod 2^32
-        const int b = (int)__double_as_longlong(__builtin_fma(w, g1_scaled, MAGIC)) + (a >> 31);
+    // The terms are turned into integers by a float FMA against 1.5 * 2^23, whose result carries the
+    // rounded product in its low mantissa bits (|term| < 2^22, which the caller's scale ensures).
+    static constexpr float MAGIC32 = 12582912.f;             // 1.5 * 2^23, bit pattern 0x4B400000
+    __device__ static inline void add2(type* p, float w, float g0_scaled, float g1_scaled) {
+        const int a = (int)(__float_as_uint(__builtin_fmaf(w, g0_scaled, MAGIC32)) - 0x4B400000u);
+        const int b = (int)(__float_as_uint(__builtin_fmaf(w, g1_scaled, MAGIC32)) - 0x4B400000u) + (a >> 31);
         const type v = ((type)(unsigned)b << 32) | (type)(unsigned)a;
         (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -857,9 +860,14 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         const bool cells_ok = bound < 3.0e38f;                        // false for NaN
         if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
         double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
+        float scale32 = 1.f;
         if constexpr (PAIR) {
-            // all the terms a cell can receive, each at the bound, stay below 2^31
-            scale = bound > 0.f && bound < 3.0e38f ? 2147483648.0 * 0.99 / ((double)(NW * TN) * P.kV * (double)bound) : 1.0;
+            // all the terms a cell can receive, each at the bound, stay below 2^31; and a single term
+            // below 2^22 (the float conversion of add2)
+            const double terms = (double)(NW * TN) * P.kV;
+            scale = bound > 0.f && bound < 3.0e38f ? 0.99 * (terms > 512.0 ? 2147483648.0 / terms : 4194304.0) / (double)bound : 1.0;
+            scale32 = (float)(scale < 1e30 ? scale : 1e30);       // (a denormal bound: keep the scale a finite float)
+            scale = (double)scale32;                 // the flush divides by exactly what the terms were multiplied with
             inv_scale = 1.0 / scale;
         }
 
@@ -1161,10 +1169,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         if constexpr (PAIR) {
 #pragma unroll
                             for (int rr = 0; rr < RPS; rr += 2) {          // consecutive registers hold consecutive channels
-                                const double g0 = LdsCell<T>::pre(gv[rr], scale), g1 = LdsCell<T>::pre(gv[rr + 1], scale);
+                                const float g0 = (float)gv[rr] * scale32, g1 = (float)gv[rr + 1] * scale32;
                                 const int pl = row_ch(ts * RPS + rr, q) / 2;
 #pragma unroll
-                                for (int i = 0; i < NC; ++i) LdsCell<T>::add2(cp + coff[i] + pl * hs, (double)cw[i], g0, g1);
+                                for (int i = 0; i < NC; ++i) LdsCell<float>::add2(cp + coff[i] + pl * hs, (float)cw[i], g0, g1);
                             }
                         } else {
 #pragma unroll
