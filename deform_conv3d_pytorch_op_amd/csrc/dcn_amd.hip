@@ -446,6 +446,13 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
             bool tiled = plan_halo<T, ND>(Ph, LDS_BUDGET, 1 << 30, sizeof(T), WAVESH, false, FQ);
             if ((!tiled || Ph.cchunk < 8) && LDS_BUDGET < 144 * 1024)
                 tiled = plan_halo<T, ND>(Ph, 144 * 1024, 1 << 30, sizeof(T), WAVESH, false, FQ) || tiled;
+            if (!tiled || Ph.cchunk < 8) {       // strided layers: the block shape with the smallest halo may hold 8 channels
+                Params Ps = P;
+                if (plan_halo<T, ND>(Ps, 144 * 1024, 1 << 30, sizeof(T), WAVESH, true, FQ) && (!tiled || Ps.cchunk > Ph.cchunk)) {
+                    Ph = Ps;
+                    tiled = true;
+                }
+            }
             if (tiled && (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks <= 0x7fffffffLL) nw = WAVESH;
         }
         const size_t slabs = (size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1;
