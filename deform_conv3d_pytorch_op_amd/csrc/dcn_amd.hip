@@ -268,6 +268,10 @@ static bool fused_pair() {              // DCN_FUSED_PAIR=0: float32 LDS cells o
     static const int v = [] { const char* e = getenv("DCN_FUSED_PAIR"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
 }
+static bool fused_breg2() {             // DCN_FUSED_BREG2=0: grad_output operand in registers only up to 32 reduction steps
+    static const int v = [] { const char* e = getenv("DCN_FUSED_BREG2"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
+}
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
     return v != 0;
@@ -599,6 +603,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         const bool wide = eight && pair && ksteps <= 32;                                         // the kernel's WIDE
         const int slot_regs = wide ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
         const bool breg = ksteps <= Mma<T>::NACC / slot_regs * (wide ? 16 : 8);
+        // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
+        const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
         {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
             const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in, cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
@@ -612,10 +618,16 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         using Kern = void (*)(Params, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
         Kern kern = nullptr;
 #define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>
+#define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2>
         auto pick = [&](auto pair_tag) {
             constexpr bool PR = decltype(pair_tag)::value;
             if (eight) {
                 if constexpr (ND == 2 || PR) kern = breg ? DCN_FUSED_C(8, true, 0, 8, PR) : DCN_FUSED_C(8, false, 0, 8, PR);
+            } else if (breg2) {
+                if constexpr (sizeof(T) == 4) {
+                    if (nw == 8) kern = fixed ? DCN_FUSED_B2(FUSED_HS, 8, PR) : DCN_FUSED_B2(0, 8, PR);
+                    else kern = fixed ? DCN_FUSED_B2(FUSED_HS, 4, PR) : DCN_FUSED_B2(0, 4, PR);
+                }
             } else if (nw == 8)
                 kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 8, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 8, PR) : DCN_FUSED_C(4, false, 0, 8, PR);
             else
@@ -626,6 +638,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             else pick(std::false_type{});
         } else
             pick(std::false_type{});
+#undef DCN_FUSED_B2
 #undef DCN_FUSED_C
         if (!kern) continue;
         if (lds > 48 * 1024)

@@ -690,8 +690,9 @@ __global__ __launch_bounds__(512) void colnorm_max_kernel(const T* __restrict__ 
 // along each axis times gcol, summed over the chunk's channels, accumulated into grad_offset
 // chunk after chunk (float atomics on a zero-filled buffer, or the first chunk stores and the
 // others add in place).  dynamic LDS then adds CCH * hstride * sizeof(T).
-// BREG = true (host: at most NS * 8 reduction steps, i.e. M <= 64 for float) keeps this lane's
-// grad_output values -- the B operand, the same for every tap and channel chunk -- in registers.
+// BREG = true (host: at most 32 * BS reduction steps, i.e. M <= 64 * BS for float) keeps this lane's
+// grad_output values -- the B operand, the same for every tap and channel chunk -- in registers;
+// the first 32 steps of a pass ride on the tap slots of the pass before, the others (BS = 2) run ahead of them.
 // NW wavefronts per workgroup (8; 4 where only a smaller block of positions has a halo that fits).
 // HS > 0 fixes the plane stride at compile time (the host then plans with hstride = HS): the plane
 // of a channel becomes an immediate offset of the LDS instructions instead of address arithmetic.
@@ -702,7 +703,7 @@ __global__ __launch_bounds__(512) void colnorm_max_kernel(const T* __restrict__ 
 // that (positions of the block x taps) of the largest possible one -- all that a cell can receive
 // -- still fit 31 bits; the host allows it only while that leaves enough bits below that term.
 // wmax[1] then holds the largest column norm of the weight (colnorm_max_kernel).
-template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false>
+template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false, int BS = 1>
 __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
@@ -796,7 +797,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         const int klast = (P.M + KL - 1) / KL - 1;
         const unsigned b_byte = b_off * (unsigned)sizeof(T);
         const unsigned b_byte_last = (klast * KL + q < P.M ? b_off : pos) * (unsigned)sizeof(T);
-        T b_reg[BREG ? NS * AB : 1];
+        T b_reg[BREG ? NS * AB * BS : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share); PAIR: of the squares
         if constexpr (BREG) {
             // held unmasked (rows past M meet zero weight rows, columns outside the volume are never
@@ -808,12 +809,12 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             asm volatile("" : "+s"(kl));
             const char* gk = reinterpret_cast<const char*>(gbase);
 #pragma unroll
-            for (int k = 0; k < NS * AB; ++k) {
+            for (int k = 0; k < NS * AB * BS; ++k) {
                 b_reg[k] = *reinterpret_cast<const T*>(gk + (k >= kl ? b_byte_last : b_byte));
                 gk += k < kl ? gstep * sizeof(T) : (size_t)0;
             }
 #pragma unroll
-            for (int k = 0; k < NS * AB; ++k) {
+            for (int k = 0; k < NS * AB * BS; ++k) {
                 const float bk = (float)b_reg[k];
                 sabs += (valid && (k < kl || (k == kl && kl * KL + q < P.M))) ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
             }
@@ -946,6 +947,21 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
+            // register-resident operand: the batches of a pass past those that ride on the tap slots
+            auto gemm_tail_reg = [&](typename MM::Acc& dd, const T* wp) {
+                if constexpr (BREG && BS > 1) {
+                    T a_x[2][AB];
+                    if (NS * AB < ksteps) load_batch(a_x[0], nullptr, wp, NS * AB);
+#pragma unroll
+                    for (int kb = NS; kb < NS * BS; ++kb) {
+                        if (kb * AB < ksteps) {
+                            if ((kb + 1) * AB < ksteps && kb + 1 < NS * BS) load_batch(a_x[(kb + 1 - NS) & 1], nullptr, wp, (kb + 1) * AB);
+#pragma unroll
+                            for (int k = 0; k < AB; ++k) dd = MM::mma(a_x[(kb - NS) & 1][k], b_reg[kb * AB + k], dd);
+                        }
+                    }
+                }
+            };
             typename MM::Acc d_next = acc_zero<T>();
             if constexpr (BREG) {                                      // first pass: nothing to hide behind
 #pragma unroll
@@ -957,6 +973,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         for (int k = 0; k < AB; ++k) d_next = MM::mma(a_cu[k], b_reg[ts * AB + k], d_next);
                     }
                 }
+                gemm_tail_reg(d_next, wchunk);
             } else {
                 gemm_tail(d_next, wchunk, 0);
             }
@@ -1036,6 +1053,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 asm volatile("" : "+s"(kz));
                 const T* wnext = wchunk + (size_t)(tap0 / TP + 1) * wpass;
                 if constexpr (!BREG) { if (more && ksteps > NS * AB) gemm_tail(d_next, wnext, NS * AB); }
+                else { if (more) gemm_tail_reg(d_next, wnext); }
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
                     // slots past the last tap (only in the last pass, which feeds no further MFMAs)

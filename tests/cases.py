@@ -64,6 +64,7 @@ SMALL_CASES = {
     "3d_k5": (3, 1, 8, 6, (6, 7, 7), 5, 1, 2, 1, 8, 1, 1.5),                  # 125 taps: too many terms per LDS cell for the paired float cells
     "2d_k7": (2, 1, 8, 10, (12, 11), 7, 1, 3, 1, 8, 1, 2.0),                   # 49 taps
     "3d_m72_chunk8": (3, 1, 16, 72, (4, 8, 9), 3, 1, 1, 1, 8, 1, 1.5),        # 36 reduction steps: the grad_output operand does not fit the registers
+    "3d_m100_chunk4": (3, 1, 8, 100, (4, 8, 9), 3, 1, 1, 1, 4, 1, 1.5),       # 50 reduction steps, 4-channel chunks: the operand takes two register sets
 }
 
 

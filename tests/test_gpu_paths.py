@@ -15,6 +15,7 @@ settings, each in a process of its own (the knobs are read once per process):
                        items of the last round split over several workgroups (otherwise only full-size layers get there)
   DCN_FUSED_TAIL=0     ... and the same without that split; DCN_FUSED_FIXED=0: runtime plane stride
   DCN_OVERLAP_BACKWARD=1  backward_weight on a second stream next to backward_input_offset
+  DCN_FUSED_BREG2=0    the grad_output operand of 64 < M <= 128 output channels read from memory instead of a second register set
   DCN_FUSED_PAIR=0     float32 LDS cells of the fused backward kernel with one channel each (64-bit) instead of two
   DCN_FORWARD_SPLIT=0  the forward pass never splits the input channels of a position block over workgroups
                        (small layers otherwise do, so the default runs cover the split and its joining kernel)
@@ -41,7 +42,7 @@ SETTINGS = [
     {"DCN_FUSED_SLOTS": "3"},
     {"DCN_FUSED_SLOTS": "3", "DCN_FUSED_TAIL": "0", "DCN_FUSED_FIXED": "0"},
     {"DCN_OVERLAP_BACKWARD": "1", "DCN_FORWARD_SPLIT": "0"},
-    {"DCN_FUSED_PAIR": "0"},
+    {"DCN_FUSED_PAIR": "0", "DCN_FUSED_BREG2": "0"},
 ]
 
 
