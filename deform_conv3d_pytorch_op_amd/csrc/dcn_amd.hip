@@ -420,7 +420,7 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
         if (tiled && forward_split() > 1 && (size_t)P.N * P.outV < FWD_SPLIT_POSITIONS && ws_bytes > wq_bound) {
             const size_t room = ws_bytes - wq_bound < FWD_PARTIAL_CAP ? ws_bytes - wq_bound : FWD_PARTIAL_CAP;
             while (fsplit * 2 <= FWD_MAX_SPLIT && fsplit * 2 <= forward_split() && tiles * P.G * P.mchunks * fsplit * 2 <= cu_count() &&
-                   (size_t)fsplit * 2 * out_bytes <= room && fsplit * 2 * FQ <= P.Cg)
+                   (size_t)fsplit * 2 * out_bytes <= room && fsplit * 2 * 16 <= P.Cg)      // at least 16 channels per part
                 fsplit *= 2;
         }
         while (MT > 1 && tiles * P.G * P.mchunks * fsplit < cu_count()) {
@@ -529,18 +529,14 @@ int absmax(const T* w, size_t n, float* out, hipStream_t s) {
     hipLaunchKernelGGL(absmax_kernel<T>, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, n, out);
     return check_launch("absmax_kernel");
 }
-// out[0] = max |w|, out[1] = largest norm over the output channels of a group of an (input channel, tap) column
+// out[0] = max |w|, out[1] = largest norm over the output channels of a group of an (input channel, tap)
+// column; `out` was cleared by the pack_weight_kernel launched before
 template <typename T>
 int weight_bounds(const Params& P, const T* w, float* out, hipStream_t s) {
-    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(1), dim3(64), 0, s, out, (size_t)2);
-    if (int rc = check_launch("fill_zero_kernel")) return rc;
-    const size_t n = (size_t)P.C_out * P.Cg * P.kV, cols = (size_t)P.Cg * P.kV;
-    const unsigned blocks = (unsigned)((n + 1023) / 1024 > 128 ? 128 : (n + 1023) / 1024);
-    hipLaunchKernelGGL(absmax_kernel<T>, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, n, out);
-    if (int rc = check_launch("absmax_kernel")) return rc;
+    const size_t cols = (size_t)P.Cg * P.kV;
     if (P.G > 65535) return fail(DCN_E_ARGUMENT, "more than 65535 convolution groups");
-    hipLaunchKernelGGL(colnorm_max_kernel<T>, dim3((unsigned)((cols + 63) / 64), (unsigned)P.G), dim3(512), 0, s, w, P.M, cols, out + 1);
-    return check_launch("colnorm_max_kernel");
+    hipLaunchKernelGGL(weight_bounds_kernel<T>, dim3((unsigned)((cols + 63) / 64), (unsigned)P.G), dim3(512), 0, s, w, P.M, cols, out);
+    return check_launch("weight_bounds_kernel");
 }
 
 template <typename T, int ND>
@@ -609,9 +605,9 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in, cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
             // (wide: row order that leaves the eight channels of a tap in one lane)
-            if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), dim3(blocks), dim3(256), 0, s, P, w, wt);
-            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), dim3(blocks), dim3(256), 0, s, P, w, wt);
-            else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt);
+            if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);
+            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);
+            else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
         if (int rc = weight_bounds<T>(P, w, wmax, s)) return rc;

@@ -50,9 +50,11 @@ __host__ __device__ inline int chunk_slot(int cpg, int Cg, int c0) { return c0 /
 // WIDE (float, CCH = 8): row j of a pass holds (tap, channel) = (2 * (j / 16) + (j / 4) % 2,
 // 4 * ((j / 8) % 2) + j % 4) instead of (j / CCH, j % CCH): the MFMA then leaves all eight channels
 // of a tap in one lane (fused_row_tap / fused_row_channel).
+// `bounds` (two floats, may be null) is cleared for the weight_bounds_kernel that follows.
 template <typename T, int CCH, bool WIDE = false>
-__global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp) {
+__global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp, float* __restrict__ bounds) {
     using MM = Mma<T>;
+    if (bounds && blockIdx.x == 0 && threadIdx.x < 2) bounds[threadIdx.x] = 0.f;
     constexpr int TN = MM::TN, KL = MM::KL, TP = TN / CCH;
     const int npass = (P.kV + TP - 1) / TP;
     const int kst = ((P.M + KL - 1) / KL + 15) / 16 * 16;       // operand batches are 8 or 16 reduction steps
@@ -639,30 +641,42 @@ __global__ void absmax_kernel(const T* __restrict__ w, size_t n, float* __restri
     if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned*>(out), redu[0]);
 }
 
-// max over the weight's (input channel, tap) columns of the Euclidean norm over the output channels
-// of one convolution group, NaN if any element is NaN: |grad column| <= that norm times the norm of
-// grad_output over the output channels at the position (Cauchy-Schwarz).  W is [G*M][Cg][kV];
-// grid (ceil(Cg*kV / 64), G); joined like absmax_kernel.  `out` must hold 0 beforehand.
+// out[0] = max |w| and out[1] = max over the weight's (input channel, tap) columns of the Euclidean
+// norm over the output channels of one convolution group, NaN if any element is NaN: |grad column|
+// <= that norm times the norm of grad_output over the output channels at the position
+// (Cauchy-Schwarz).  W is [G*M][Cg][kV]; grid (ceil(Cg*kV / 64), G); joined like absmax_kernel.
+// `out` must hold two zeros beforehand.
 template <typename T>
-__global__ __launch_bounds__(512) void colnorm_max_kernel(const T* __restrict__ w, int M, size_t cols, float* __restrict__ out) {
+__global__ __launch_bounds__(512) void weight_bounds_kernel(const T* __restrict__ w, int M, size_t cols, float* __restrict__ out) {
     // workgroup = 64 neighbouring columns of one group (blockIdx.y) x 8 slices of its rows
     __shared__ float part[8][64];
+    __shared__ unsigned amax[8];
     const int cx = threadIdx.x & 63, sl = threadIdx.x >> 6;
     const size_t col = (size_t)blockIdx.x * 64 + cx;
     float ss = 0.f;
+    unsigned am = 0u;
     if (col < cols) {
         const T* p = w + (size_t)blockIdx.y * M * cols + col;
 #pragma unroll 8
-        for (int r = sl; r < M; r += 8) { const float v = (float)p[(size_t)r * cols]; ss += v * v; }
+        for (int r = sl; r < M; r += 8) {
+            const float v = (float)p[(size_t)r * cols];
+            ss += v * v;
+            am = max(am, __float_as_uint(fabsf(v)));
+        }
     }
+    for (int sh = 1; sh < 64; sh <<= 1) am = max(am, (unsigned)__shfl_xor((int)am, sh));
     part[sl][cx] = ss;
+    if (cx == 0) amax[sl] = am;
     __syncthreads();
     if (sl == 0) {
 #pragma unroll
-        for (int k = 1; k < 8; ++k) ss += part[k][cx];
+        for (int k = 1; k < 8; ++k) { ss += part[k][cx]; am = max(am, amax[k]); }
         unsigned m = __float_as_uint(fabsf(sqrtf(ss)));       // NaN keeps the largest pattern
         for (int sh = 1; sh < 64; sh <<= 1) m = max(m, (unsigned)__shfl_xor((int)m, sh));
-        if (cx == 0) atomicMax(reinterpret_cast<unsigned*>(out), m);
+        if (cx == 0) {
+            atomicMax(reinterpret_cast<unsigned*>(out), am);          // out[0] = max |w|
+            atomicMax(reinterpret_cast<unsigned*>(out) + 1, m);       // out[1] = largest column norm
+        }
     }
 }
 

@@ -99,7 +99,7 @@ def _geom(nd, inputs, weight, out_sizes, stride, padding, dilation, channel_per_
             list(weight.shape[2:]) + list(padding) + list(stride) + list(dilation) + [channel_per_group, group])
 
 
-def _workspace(inputs, weight, group, out_sizes, channel_per_group):
+def _workspace_bytes(inputs, weight, group, out_sizes, channel_per_group):
     L = _lib.load()
     kV = inV = outV = 1
     for k in weight.shape[2:]:
@@ -108,13 +108,33 @@ def _workspace(inputs, weight, group, out_sizes, channel_per_group):
         inV *= v
     for v in out_sizes:
         outV *= v
-    nbytes = L.dcn_workspace_bytes_for(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, outV,
-                                       kV, group, channel_per_group)
-    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=inputs.device), int(nbytes)
+    return int(L.dcn_workspace_bytes_for(inputs.element_size(), inputs.size(0), inputs.size(1), weight.size(0), inV, outV,
+                                         kV, group, channel_per_group))
+
+
+def _workspace(inputs, weight, group, out_sizes, channel_per_group):
+    nbytes = _workspace_bytes(inputs, weight, group, out_sizes, channel_per_group)
+    return torch.empty(max(nbytes, 1), dtype=torch.uint8, device=inputs.device), nbytes
 
 
 def _stream():
     return torch.cuda.current_stream().cuda_stream
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` only when d is not the current device (the context manager costs
+    several microseconds, which shows on small layers)."""
+
+    def __init__(self, device):
+        self.ctx = None if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
 
 
 # DCN_OVERLAP_BACKWARD=1: backward_weight next to backward_input_offset on a second stream (default: one stream)
@@ -130,26 +150,47 @@ def _side_stream(device):
     return _SIDE_STREAMS[key]
 
 
+# Checked layer geometries: (output sizes, the C ABI's geometry arguments, workspace bytes) per
+# (shapes, dtype, parameters).  A layer that passed the shape checks once skips them afterwards.
+_PLANS = {}
+
+
+def _plan(nd, inputs, offset, weight, out_shape, stride, padding, dilation, channel_per_group, group, standard):
+    key = (nd, inputs.dtype, inputs.shape, offset.shape, weight.shape, out_shape, stride, padding, dilation,
+           channel_per_group, group, standard)
+    plan = _PLANS.get(key)
+    if plan is None:
+        _check(inputs.dim() == nd + 2, "input dim")
+        _check(weight.dim() == nd + 2, "kernel dim")
+        outs = output_size(inputs.shape[2:], weight.shape[2:], stride, padding, dilation, standard)
+        shape = (inputs.size(0), weight.size(0)) + outs if out_shape is None else tuple(out_shape)
+        shape_check(nd, inputs, weight, offset, shape, channel_per_group, group, stride, padding, dilation, standard)
+        outs = tuple(shape[2:])
+        plan = (shape, tuple(_geom(nd, inputs, weight, outs, stride, padding, dilation, channel_per_group, group)),
+                _workspace_bytes(inputs, weight, group, outs, channel_per_group))
+        if len(_PLANS) > 4096:
+            _PLANS.clear()
+        _PLANS[key] = plan
+    return plan
+
+
 def _forward(nd, inputs, offset, weight, bias, stride, padding, dilation, channel_per_group, group, standard=False):
     L = _lib.load()
     stride, padding, dilation = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
     _device_check(inputs, offset, weight, bias)
-    _check(inputs.dim() == nd + 2, "input dim")
-    _check(weight.dim() == nd + 2, "kernel dim")
-    outs = output_size(inputs.shape[2:], weight.shape[2:], stride, padding, dilation, standard)
-    out_shape = (inputs.size(0), weight.size(0)) + outs
-    shape_check(nd, inputs, weight, offset, out_shape, channel_per_group, group, stride, padding, dilation, standard)
+    out_shape, geom, ws_bytes = _plan(nd, inputs, offset, weight, None, stride, padding, dilation, channel_per_group, group,
+                                      standard)
     if bias is not None:
         _check(bias.dim() == 1 and bias.size(0) == weight.size(0), "bias size")
     inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
-    output = torch.empty(out_shape, dtype=inputs.dtype, device=inputs.device)
-    ws, ws_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
+    device = inputs.device
+    output = torch.empty(out_shape, dtype=inputs.dtype, device=device)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device)
     fn = getattr(L, "dcn%dd_forward_%s" % (nd, _SUFFIX[inputs.dtype]))
-    with torch.cuda.device(inputs.device):
+    with _on_device(device):
         rc = fn(inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(),
                 bias.contiguous().data_ptr() if bias is not None else None, output.data_ptr(),
-                *_geom(nd, inputs, weight, outs, stride, padding, dilation, channel_per_group, group),
-                ws.data_ptr(), ws_bytes, _stream())
+                *geom, ws.data_ptr(), ws_bytes, torch.cuda.current_stream(device).cuda_stream)
     _lib.check(rc)
     return output
 
@@ -158,28 +199,27 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
               need_data, need_weight, standard=False, oob_zero=False):
     L = _lib.load()
     _device_check(inputs, offset, weight, grad_output)
-    outs = tuple(grad_output.shape[2:])
-    shape_check(nd, inputs, weight, offset, tuple(grad_output.shape), channel_per_group, group, stride, padding,
-                dilation, standard)
+    _, geom, ws_bytes = _plan(nd, inputs, offset, weight, grad_output.shape, stride, padding, dilation, channel_per_group,
+                              group, standard)
     inputs, offset, weight = inputs.contiguous(), offset.contiguous(), weight.contiguous()
     grad_output = grad_output.contiguous()
-    geom = _geom(nd, inputs, weight, outs, stride, padding, dilation, channel_per_group, group)
     suf = _SUFFIX[inputs.dtype]
+    device = inputs.device
     grad_input = grad_offset = grad_weight = None
-    with torch.cuda.device(inputs.device):
-        main = torch.cuda.current_stream()
+    with _on_device(device):
+        main = torch.cuda.current_stream(device)
         # The two backward calls are independent.  On request (DCN_OVERLAP_BACKWARD=1) backward_weight
         # runs on a second stream of the same priority with a workspace of its own.  It is off by
         # default: a workgroup of the fused backward kernel takes nearly all of a CU's LDS, so the
         # two kernels never share a CU; they only take turns, which upsets the order in which the
         # fused kernel works through its items (whole rounds first, split items last) and measured
         # slower than one stream (4.02 against 3.69 ms per step at 64 -> 64 channels, 16x56x56).
-        side = _side_stream(inputs.device) if (need_data and need_weight and _OVERLAP_BACKWARD) else None
+        side = _side_stream(device) if (need_data and need_weight and _OVERLAP_BACKWARD) else None
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device)
+        ws_w = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device) if side is not None else ws
         if need_weight:
             grad_weight = torch.zeros_like(weight)          # beta = 1 accumulation, as in the reference
-            ws_w, ws_w_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
         if need_data:
-            ws, ws_bytes = _workspace(inputs, weight, group, outs, channel_per_group)
             # the kernels accumulate into grad_input (as the reference's atomicAdd does) and store
             # every element of grad_offset
             grad_input = torch.zeros_like(inputs)
@@ -187,8 +227,6 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
         if side is not None:
             side.wait_stream(main)           # the operands and the zero fills above are ready
         if need_data:
-            # issued first: its one large workgroup per CU takes its place and the small workgroups of
-            # backward_weight fill what is left, instead of the other way round
             args = (inputs.data_ptr(), weight.data_ptr(), offset.data_ptr(), grad_output.data_ptr(),
                     grad_input.data_ptr(), grad_offset.data_ptr(), *geom, ws.data_ptr(), ws_bytes, main.cuda_stream)
             if nd == 3 and oob_zero:        # the reference's 2-D kernels have no out-of-range term
@@ -199,7 +237,7 @@ def _backward(nd, inputs, offset, weight, grad_output, stride, padding, dilation
         if need_weight:
             fn = getattr(L, "dcn%dd_backward_weight_%s" % (nd, suf))
             _lib.check(fn(inputs.data_ptr(), offset.data_ptr(), grad_output.data_ptr(), grad_weight.data_ptr(),
-                          *geom, ws_w.data_ptr(), ws_w_bytes, (side or main).cuda_stream))
+                          *geom, ws_w.data_ptr(), ws_bytes, (side or main).cuda_stream))
         if side is not None:
             main.wait_stream(side)           # everything issued later on the caller's stream sees grad_weight
     return grad_input, grad_offset, grad_weight
