@@ -477,7 +477,7 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
                     if (chunks_of_group0(cc) % fsplit == 0) { Ph.cchunk = cc; break; }
             }
             {
-                const size_t total = (size_t)P.C_in * forward_slab_elems<T>(P.kV, P.Mp);
+                const size_t total = (size_t)chunk_candidates<FQ>(P.cpg, P.Cg, P.C_in) * forward_slab_elems<T>(P.kV, P.Mp);
                 const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
                 hipLaunchKernelGGL(pack_forward_weight_kernel<T>, dim3(blocks), dim3(256), 0, s, Ph, w, wt);
                 if (int rc = check_launch("pack_forward_weight_kernel")) return rc;
@@ -602,7 +602,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
         const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
         {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
-            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)P.C_in, cch);
+            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)(eight ? chunk_candidates<8>(P.cpg, P.Cg, P.C_in)
+                                                                                      : chunk_candidates<4>(P.cpg, P.Cg, P.C_in)), cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
             // (wide: row order that leaves the eight channels of a tap in one lane)
             if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);

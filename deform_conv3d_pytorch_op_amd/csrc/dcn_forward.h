@@ -36,9 +36,9 @@ __global__ void pack_forward_weight_kernel(Params P, const T* __restrict__ W, T*
     constexpr int TN = MM::TN, KL = MM::KL;
     const int mtiles = P.Mp / TN;
     const size_t per_slab = forward_slab_elems<T>(P.kV, P.Mp);
-    const size_t total = (size_t)P.C_in * per_slab;
+    const size_t total = (size_t)chunk_candidates<FQ>(P.cpg, P.Cg, P.C_in) * per_slab;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const int c0 = (int)(i / per_slab);                    // candidate first channel of a group
+        const int c0 = chunk_candidate<FQ>(P.cpg, P.Cg, (int)(i / per_slab));       // candidate first channel of a group
         const int seg_b = max(c0 / P.cpg * P.cpg, c0 / P.Cg * P.Cg);
         if ((c0 - seg_b) % FQ) continue;
         const int seg_e = min((c0 / P.cpg + 1) * P.cpg, (c0 / P.Cg + 1) * P.Cg);

@@ -46,6 +46,21 @@ __global__ void relayout_weight_kernel(Params P, const T* __restrict__ W, T* __r
 // chunks share a slab; some slabs stay unused.
 template <int CCH>
 __host__ __device__ inline int chunk_slot(int cpg, int Cg, int c0) { return c0 / CCH + c0 / cpg + c0 / Cg; }
+// The pack kernels walk over candidate chunk starts.  Where one of cpg and Cg divides the other
+// (nearly every layer) the segments all have the length of the smaller and the y-th chunk start
+// is known in closed form; otherwise every channel is a candidate and non-starts are skipped.
+template <int CCH>
+__host__ __device__ inline int chunk_candidates(int cpg, int Cg, int C_in) {
+    const int seg = cpg < Cg ? cpg : Cg, big = cpg < Cg ? Cg : cpg;
+    return big % seg == 0 ? C_in / seg * ((seg + CCH - 1) / CCH) : C_in;
+}
+template <int CCH>
+__host__ __device__ inline int chunk_candidate(int cpg, int Cg, int y) {     // first channel of candidate y
+    const int seg = cpg < Cg ? cpg : Cg, big = cpg < Cg ? Cg : cpg;
+    if (big % seg) return y;
+    const int cps = (seg + CCH - 1) / CCH;
+    return y / cps * seg + y % cps * CCH;
+}
 
 // WIDE (float, CCH = 8): row j of a pass holds (tap, channel) = (2 * (j / 16) + (j / 4) % 2,
 // 4 * ((j / 8) % 2) + j % 4) instead of (j / CCH, j % CCH): the MFMA then leaves all eight channels
@@ -59,9 +74,9 @@ __global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restr
     const int npass = (P.kV + TP - 1) / TP;
     const int kst = ((P.M + KL - 1) / KL + 15) / 16 * 16;       // operand batches are 8 or 16 reduction steps
     const size_t per_chunk = (size_t)npass * kst * 64;
-    const size_t total = (size_t)P.C_in * per_chunk;
+    const size_t total = (size_t)chunk_candidates<CCH>(P.cpg, P.Cg, P.C_in) * per_chunk;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const int c0 = (int)(i / per_chunk);                    // candidate first channel of a chunk
+        const int c0 = chunk_candidate<CCH>(P.cpg, P.Cg, (int)(i / per_chunk));      // candidate first channel of a chunk
         const int seg_b = max(c0 / P.cpg * P.cpg, c0 / P.Cg * P.Cg);
         if ((c0 - seg_b) % CCH) continue;
         const int seg_e = min((c0 / P.cpg + 1) * P.cpg, (c0 / P.Cg + 1) * P.Cg);
