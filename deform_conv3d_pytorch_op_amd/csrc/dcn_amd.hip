@@ -272,6 +272,10 @@ static bool fused_breg2() {             // DCN_FUSED_BREG2=0: grad_output operan
     static const int v = [] { const char* e = getenv("DCN_FUSED_BREG2"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
 }
+static bool native16() {                // DCN_NATIVE16=0: the 16-bit forward entry points always widen to float32 first
+    static const int v = [] { const char* e = getenv("DCN_NATIVE16"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
+}
 static bool scatter_in_lds() {
     static const int v = [] { const char* e = getenv("DCN_SCATTER"); return (e && strcmp(e, "global") == 0) ? 0 : 1; }();
     return v != 0;
@@ -386,17 +390,22 @@ int launch_halo(K kern, const char* name, dim3 grid, int threads, size_t lds, hi
     return check_launch(name);
 }
 
-template <typename T, int ND>
-int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* bias, T* out, void* ws,
-            size_t ws_bytes, hipStream_t s) {
+// S = T: the float32 / float64 operator.  S = Bf16 / Fp16 (T = float): the tensors are in that
+// storage format and only the LDS-halo kernel serves them; where it cannot (halo too large, a layer
+// that wants the input-channel split), *declined is set and nothing is launched: the caller then
+// widens the tensors and runs the float32 operator.
+template <typename T, int ND, typename S = T>
+int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* bias, S* out, void* ws,
+            size_t ws_bytes, hipStream_t s, bool* declined = nullptr) {
+    constexpr bool S16 = !std::is_same<S, T>::value;
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (!in || !w || !off || !out) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     if (int rc = device_info(nullptr)) return rc;
     int MT;
     fwd_weight_pad<T>(P.M, P.Cg, MT, P.mchunks, P.Mp, P.Cgp);
-    if (!ws || ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T)) return fail(DCN_E_WORKSPACE, "workspace too small");
-    T* wt = static_cast<T*>(ws);
+    if (!ws || (!S16 && ws_bytes < (size_t)P.G * P.kV * P.Mp * P.Cgp * sizeof(T))) return fail(DCN_E_WORKSPACE, "workspace too small");
+    S* wt = static_cast<S*>(ws);
     const int TN = Mma<T>::TN;
     // Too few position blocks to give every CU a workgroup.  First the input channels of a block are
     // split over up to FWD_MAX_SPLIT workgroups (each samples its own channels once; their partial
@@ -417,7 +426,7 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
             MT = 4;
             P.mchunks = (mtiles_all + MT - 1) / MT;
         }
-        if (tiled && forward_split() > 1 && (size_t)P.N * P.outV < FWD_SPLIT_POSITIONS && ws_bytes > wq_bound) {
+        if (!S16 && tiled && forward_split() > 1 && (size_t)P.N * P.outV < FWD_SPLIT_POSITIONS && ws_bytes > wq_bound) {
             const size_t room = ws_bytes - wq_bound < FWD_PARTIAL_CAP ? ws_bytes - wq_bound : FWD_PARTIAL_CAP;
             while (fsplit * 2 <= FWD_MAX_SPLIT && fsplit * 2 <= forward_split() && tiles * P.G * P.mchunks * fsplit * 2 <= cu_count() &&
                    (size_t)fsplit * 2 * out_bytes <= room && fsplit * 2 * 16 <= P.Cg)      // at least 16 channels per part
@@ -460,7 +469,7 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
             if (tiled && (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks <= 0x7fffffffLL) nw = WAVESH;
         }
         const size_t slabs = (size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1;
-        const size_t wq_bytes = slabs * forward_slab_elems<T>(P.kV, P.Mp) * sizeof(T);
+        const size_t wq_bytes = slabs * forward_slab_elems<T>(P.kV, P.Mp) * sizeof(S);
         if (nw == 16 || ws_bytes < align256(wq_bytes) + (size_t)fsplit * out_bytes) fsplit = 1;
         if (nw && ws_bytes >= wq_bytes) {
             if (fsplit > 1) {
@@ -479,33 +488,39 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
             {
                 const size_t total = (size_t)chunk_candidates<FQ>(P.cpg, P.Cg, P.C_in) * forward_slab_elems<T>(P.kV, P.Mp);
                 const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
-                hipLaunchKernelGGL(pack_forward_weight_kernel<T>, dim3(blocks), dim3(256), 0, s, Ph, w, wt);
+                hipLaunchKernelGGL((pack_forward_weight_kernel<T, S>), dim3(blocks), dim3(256), 0, s, Ph, w, wt);
                 if (int rc = check_launch("pack_forward_weight_kernel")) return rc;
             }
             const size_t lds = (size_t)Ph.cchunk * Ph.hstride * sizeof(T) + (size_t)Ph.hvol * 4;
             const dim3 grid((unsigned)Ph.N * Ph.tiles * Ph.G * Ph.mchunks * fsplit);
-            T* part = reinterpret_cast<T*>(static_cast<char*>(ws) + align256(wq_bytes));
-            T* dst = fsplit > 1 ? part : out;
-            const T* kbias = fsplit > 1 ? nullptr : bias;
+            S* part = reinterpret_cast<S*>(static_cast<char*>(ws) + align256(wq_bytes));
+            S* dst = fsplit > 1 ? part : out;
+            const S* kbias = fsplit > 1 ? nullptr : bias;
             int rc;
             if (nw == 16) {
-                rc = MT == 1 ? launch_halo(forward_quad_kernel<T, ND, 1, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit)
-                             : launch_halo(forward_quad_kernel<T, ND, 2, 16>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit);
+                rc = MT == 1 ? launch_halo(forward_quad_kernel<T, ND, 1, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit)
+                             : launch_halo(forward_quad_kernel<T, ND, 2, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit);
             } else {
                 switch (MT) {
-                    case 1: rc = launch_halo(forward_quad_kernel<T, ND, 1, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
-                    case 2: rc = launch_halo(forward_quad_kernel<T, ND, 2, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
-                    case 4: rc = launch_halo(forward_quad_kernel<T, ND, 4, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
-                    default: rc = launch_halo(forward_quad_kernel<T, ND, 8, WAVESH>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    case 1: rc = launch_halo(forward_quad_kernel<T, ND, 1, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    case 2: rc = launch_halo(forward_quad_kernel<T, ND, 2, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    case 4: rc = launch_halo(forward_quad_kernel<T, ND, 4, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    default: rc = launch_halo(forward_quad_kernel<T, ND, 8, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
                 }
             }
             if (rc || fsplit == 1) return rc;
-            const size_t total = (size_t)P.N * P.C_out * P.outV;
-            const unsigned jb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
-            hipLaunchKernelGGL(forward_join_partials_kernel<T>, dim3(jb), dim3(256), 0, s, part, bias, out, fsplit, total, P.C_out, P.outV);
-            return check_launch("forward_join_partials_kernel");
+            if constexpr (!S16) {
+                const size_t total = (size_t)P.N * P.C_out * P.outV;
+                const unsigned jb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+                hipLaunchKernelGGL(forward_join_partials_kernel<T>, dim3(jb), dim3(256), 0, s, part, bias, out, fsplit, total, P.C_out, P.outV);
+                return check_launch("forward_join_partials_kernel");
+            }
         }
     }
+    if constexpr (S16) {
+        if (declined) *declined = true;
+        return DCN_OK;
+    } else {
     if (int rc = relayout<T>(P, w, wt, 0, s)) return rc;
     // geometry whose halo does not fit in LDS: gather straight from global memory
     P.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
@@ -519,6 +534,7 @@ int forward(const Geometry& g, const T* in, const T* w, const T* off, const T* b
         default: hipLaunchKernelGGL((forward_kernel<T, ND, 8>), grid, dim3(WG), 0, s, P, in, off, wt, bias, out); break;
     }
     return check_launch("forward_kernel");
+    }
 }
 
 template <typename T>
@@ -892,6 +908,11 @@ int forward16(const Geometry& g, const S* in, const S* w, const S* off, const S*
     if (int rc = validate(g, P)) return rc;
     if (!in || !w || !off || !out) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     if (int rc = device_info(nullptr)) return rc;
+    if (native16()) {       // the LDS-halo kernel reads the 16-bit tensors itself and multiplies with 16-bit matrix instructions
+        bool declined = false;
+        if (int rc = forward<float, ND, S>(g, in, w, off, bias, out, ws, ws_bytes, s, &declined)) return rc;
+        if (!declined) return DCN_OK;
+    }
     const Sizes16 z = sizes16(P, ND);
     Carver c{static_cast<char*>(ws), ws ? ws_bytes : 0};
     float *fin = c.take(z.in), *fw = c.take(z.w), *foff = c.take(z.off), *fout = c.take(z.out), *fb = bias ? c.take(P.C_out) : nullptr;

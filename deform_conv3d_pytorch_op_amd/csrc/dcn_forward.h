@@ -15,9 +15,41 @@
 #pragma once
 #include "dcn_kernels.h"
 
+#include <type_traits>
+
 namespace dcn {
 
 constexpr int FQ = 4;              // channels per group: one wide LDS read per corner
+
+// Storage format of the tensors in global memory.  float / double: the arithmetic type itself.
+// Bf16 / Fp16: 16-bit storage, float arithmetic; the sampled columns and the weights then meet in
+// v_mfma_f32_32x32x8_bf16 / _f16 (float accumulation), a quarter of the matrix instructions.
+template <typename S> struct Store { static __device__ inline S ld(S v) { return v; } static __device__ inline S st(S v) { return v; } };
+template <> struct Store<Bf16> {
+    static __device__ inline float ld(Bf16 v) { return Bf16::widen(v); }
+    static __device__ inline Bf16 st(float v) { return Bf16::narrow(v); }
+};
+template <> struct Store<Fp16> {
+    static __device__ inline float ld(Fp16 v) { return Fp16::widen(v); }
+    static __device__ inline Fp16 st(float v) { return Fp16::narrow(v); }
+};
+typedef short Short4 __attribute__((ext_vector_type(4)));
+typedef _Float16 Half4 __attribute__((ext_vector_type(4)));
+typedef __bf16 Bfloat4 __attribute__((ext_vector_type(4)));
+template <typename S> struct Mma16;
+template <> struct Mma16<Bf16> {
+    typedef Short4 Vec;
+    static __device__ inline Vec pack(const float v[4]) {
+        const Bfloat4 b = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};      // round to nearest even
+        return __builtin_bit_cast(Short4, b);
+    }
+    static __device__ inline Mma<float>::Acc mma(Vec a, Vec b, Mma<float>::Acc c) { return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a, b, c, 0, 0, 0); }
+};
+template <> struct Mma16<Fp16> {
+    typedef Half4 Vec;
+    static __device__ inline Vec pack(const float v[4]) { return Vec{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]}; }
+    static __device__ inline Mma<float>::Acc mma(Vec a, Vec b, Mma<float>::Acc c) { return __builtin_amdgcn_mfma_f32_32x32x8f16(a, b, c, 0, 0, 0); }
+};
 
 // Weights of the forward kernel: one slab per group of four channels (groups start at the first
 // channel of a segment -- the channels shared by one deformable group and one convolution group --
@@ -30,8 +62,8 @@ __host__ __device__ inline size_t forward_slab_elems(int kV, int Mp) {
     return (size_t)((kV + Mma<T>::KL - 1) / Mma<T>::KL) * Mp * Mma<T>::KL * FQ;
 }
 
-template <typename T>
-__global__ void pack_forward_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wq) {
+template <typename T, typename S = T>
+__global__ void pack_forward_weight_kernel(Params P, const S* __restrict__ W, S* __restrict__ Wq) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL;
     const int mtiles = P.Mp / TN;
@@ -49,7 +81,7 @@ __global__ void pack_forward_weight_kernel(Params P, const T* __restrict__ W, T*
         const int tile = (int)(r % mtiles);
         const int tg = (int)(r / mtiles);
         const int m = tile * TN + j, tap = tg * KL + q, c = c0 + e, g = c0 / P.Cg;
-        T v = 0;
+        S v = S();
         if (m < P.M && tap < P.kV && c < seg_e) v = W[(((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap];
         Wq[(size_t)chunk_slot<FQ>(P.cpg, P.Cg, c0) * per_slab + i % per_slab] = v;
     }
@@ -58,8 +90,8 @@ __global__ void pack_forward_weight_kernel(Params P, const T* __restrict__ W, T*
 // Stage `nch` channels of the halo as groups of four: sIn[group][halo voxel][4].  Missing channels
 // of a short last group and halo voxels outside the volume hold zero (a sample in the rim reads
 // the latter with weight zero).
-template <typename T, int WGS>
-__device__ inline void halo_stage_quads(const Params& P, const T* __restrict__ chan0, int nch,
+template <typename T, int WGS, typename S = T>
+__device__ inline void halo_stage_quads(const Params& P, const S* __restrict__ chan0, int nch,
                                         const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
     const int ngrp = (nch + FQ - 1) / FQ;
     for (int v = threadIdx.x; v < P.hvol; v += WGS) {
@@ -68,7 +100,7 @@ __device__ inline void halo_stage_quads(const Params& P, const T* __restrict__ c
         for (int grp = 0; grp < ngrp; ++grp) {
             T val[FQ];
 #pragma unroll
-            for (int e = 0; e < FQ; ++e) val[e] = chan0[(size_t)min(grp * FQ + e, nch - 1) * P.inV + g];
+            for (int e = 0; e < FQ; ++e) val[e] = Store<S>::ld(chan0[(size_t)min(grp * FQ + e, nch - 1) * P.inV + g]);
 #pragma unroll
             for (int e = 0; e < FQ; ++e)
                 sIn[((size_t)grp * P.hstride + v) * FQ + e] = (grp * FQ + e < nch && t != ~0u) ? val[e] : (T)0;
@@ -84,12 +116,14 @@ __device__ inline void halo_stage_quads(const Params& P, const T* __restrict__ c
 // forward_join_partials_kernel adds them up in a fixed order.
 // (few accumulators: four wavefronts per SIMD, i.e. at most 128 registers, also for the 512-thread
 // shape, so that two of its workgroups share a CU)
-template <typename T, int ND, int MT, int NW>
-__global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, const T* __restrict__ in,
-                                                           const T* __restrict__ off, const T* __restrict__ Wq,
-                                                           const T* __restrict__ bias, T* __restrict__ out, int csplit) {
+// S: storage format of the tensors (see Store); with a 16-bit format T is float and csplit must be 1.
+template <typename T, int ND, int MT, int NW, typename S = T>
+__global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, const S* __restrict__ in,
+                                                           const S* __restrict__ off, const S* __restrict__ Wq,
+                                                           const S* __restrict__ bias, S* __restrict__ out, int csplit) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, WGS = NW * 64;
+    constexpr bool S16 = sizeof(S) == 2;                // 16-bit storage: 16-bit matrix instructions
     typedef T V4 __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sIn = reinterpret_cast<T*>(smem_raw);                                            // [cchunk / 4][hstride][4]
@@ -138,28 +172,28 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     int chunk_no = 0;
     for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
         const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
-        const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+        const S* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
         for (int cc0 = cb; cc0 < ce; cc0 += P.cchunk) {
             if ((chunk_no++) % csplit != cz) continue;                     // another workgroup's chunk (uniform)
             const int nch = min(P.cchunk, ce - cc0);
             const int ngrp = (nch + FQ - 1) / FQ;
-            const T* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
+            const S* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
             __syncthreads();                                               // readers of the previous chunk are done
-            halo_stage_quads<T, WGS>(P, chan0, nch, sTab, sIn);
+            halo_stage_quads<T, WGS, S>(P, chan0, nch, sTab, sIn);
             __syncthreads();
             // slabs of consecutive groups of one segment are consecutive.  Uniform base (scalar
             // registers); the lanes add the 32-bit offset w_lane.
-            const T* wchunk = Wq + (size_t)chunk_slot<FQ>(P.cpg, P.Cg, cc0) * per_slab;
+            const S* wchunk = Wq + (size_t)chunk_slot<FQ>(P.cpg, P.Cg, cc0) * per_slab;
 
             // kernel coordinates of this lane's tap, counted up with the tap groups
             int kq[ND];
             decode_tap<ND>(P, q, kq);
             T o_buf[2][ND];
             auto load_offsets_of = [&](int tgi, T* dst) {                  // offsets of tap tgi*KL + q (clamped to a legal tap)
-                const T* ob = off_dg + (size_t)tgi * KL * ND * P.outV;     // uniform
+                const S* ob = off_dg + (size_t)tgi * KL * ND * P.outV;     // uniform
                 const unsigned lo = (unsigned)min(q, P.kV - 1 - tgi * KL) * ND * P.outV + pos;
 #pragma unroll
-                for (int a = 0; a < ND; ++a) dst[a] = (ob + (size_t)a * P.outV)[lo];
+                for (int a = 0; a < ND; ++a) dst[a] = Store<S>::ld((ob + (size_t)a * P.outV)[lo]);
             };
             load_offsets_of(0, o_buf[0]);
 
@@ -219,11 +253,13 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
                     kq[0] += carry;
                 }
                 const V4* hp = reinterpret_cast<const V4*>(sIn) + base;
-                const T* wp = wchunk + (size_t)tgi * w_tg;
+                const S* wp = wchunk + (size_t)tgi * w_tg;
                 for (int grp = 0; grp < ngrp; ++grp) {
-                    V4 a4[MT];
+                    // this lane's weights of the group's four channels: one 16- (32-, 8-) byte load per row tile
+                    typedef typename std::conditional<S16, typename Mma16<typename std::conditional<S16, S, Bf16>::type>::Vec, V4>::type A4;
+                    A4 a4[MT];
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) a4[mt] = *reinterpret_cast<const V4*>(wp + (w_lane + mt * w_tile));
+                    for (int mt = 0; mt < MT; ++mt) a4[mt] = *reinterpret_cast<const A4*>(wp + (w_lane + mt * w_tile));
                     // weighted corner sum, four corners at a time (all eight in flight would cost 32
                     // registers that the 16-wavefront shape does not have)
                     // (element by element: a vector times scalar product would hold four copies of
@@ -251,11 +287,22 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
 #pragma unroll
                             for (int i = 0; i < 4; ++i) val[e] += c4[i][e] * cw[4 + i];
                     }
+                    if constexpr (S16) {
+                        // the four channels are the four reduction elements this lane supplies to one
+                        // 32x32x8 instruction (lane group q: elements 4q .. 4q + 3, its tap)
+                        float b4[FQ];
 #pragma unroll
-                    for (int e = 0; e < FQ; ++e) {
-                        const T b = near ? val[e] : (T)0;
+                        for (int e = 0; e < FQ; ++e) b4[e] = near ? val[e] : 0.f;
+                        const auto bv = Mma16<S>::pack(b4);
 #pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a4[mt][e], b, acc[mt]);
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = Mma16<S>::mma(a4[mt], bv, acc[mt]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < FQ; ++e) {
+                            const T b = near ? val[e] : (T)0;
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a4[mt][e], b, acc[mt]);
+                        }
                     }
                     hp += P.hstride;
                     wp += per_slab;
@@ -273,13 +320,20 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
                         t.f[a] = pa - (T)l;
                     }
                     tap_corner_idx<T, ND>(P, t);
-                    const T* wf = wchunk + (size_t)tgi * w_tg;
+                    const S* wf = wchunk + (size_t)tgi * w_tg;
                     for (int c = 0; c < nch; ++c) {
                         T b = 0;
-                        if (far) b = sample<T, ND>(chan0 + (size_t)c * P.inV, t.idx, t.f);
-                        const T* wc = wf + (size_t)(c / FQ) * per_slab + c % FQ;
+                        if (far) {
+                            T cc[NC];
 #pragma unroll
-                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(wc[w_lane + mt * w_tile], b, acc[mt]);
+                            for (int i = 0; i < NC; ++i) cc[i] = Store<S>::ld((chan0 + (size_t)c * P.inV)[t.idx[i]]);
+                            b = interp<T, ND>(cc, t.f);
+                            if constexpr (S16) b = Store<S>::ld(Store<S>::st(b));      // rounded like the samples of the halo path
+                        }
+                        const S* wc = wf + (size_t)(c / FQ) * per_slab + c % FQ;
+                        // (one channel at a time through the float instruction: same accumulator layout)
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma((T)Store<S>::ld(wc[w_lane + mt * w_tile]), b, acc[mt]);
                     }
                 }
             };
@@ -297,7 +351,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     }
 
     if (!valid) return;
-    T* dst = out + (size_t)cz * P.N * P.C_out * P.outV;
+    S* dst = out + (size_t)cz * P.N * P.C_out * P.outV;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -305,8 +359,8 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
             const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
             if (m < P.M) {
                 T v = acc[mt][r];
-                if (bias) v += bias[g * P.M + m];
-                dst[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+                if (bias) v += Store<S>::ld(bias[g * P.M + m]);
+                dst[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = Store<S>::st(v);
             }
         }
 }

@@ -163,16 +163,21 @@ int dcn2d_backward_weight_f64(const double *input, const double *offset, const d
                               double *grad_weight, DCN2D_GEOMETRY, void *workspace,
                               size_t workspace_bytes, void *stream);
 
-/* ---- 16-bit storage, float32 arithmetic ------------------------------------------------------
+/* ---- 16-bit storage, float32 accumulation ----------------------------------------------------
  * No counterpart in the reference, which instantiates float only
  * (deform3d/lib/deform_conv3d_cuda_kernel.cu:162-172).  Every tensor (input, weight, offset, bias,
- * grad_output and the results) is stored as bfloat16 (_bf16) or IEEE binary16 (_f16); the values are
- * widened exactly, all products and sums are the float32 kernels', and each result element is
- * rounded once, to nearest even.  Same argument meaning and accumulate / overwrite contract as
- * the _f32 calls (grad_input and grad_weight: rounded sum of their previous content and the
- * gradient).  The workspace must come from dcn_workspace_bytes_for(2, ...): it also holds float
- * copies of the tensors.  Offsets in 16 bits limit the sampling positions to that format's grid
- * (bfloat16: 1/128 voxel between 1 and 2, coarser above). */
+ * grad_output and the results) is stored as bfloat16 (_bf16) or IEEE binary16 (_f16).
+ * forward: coordinates and interpolation in float32; the sampled columns are rounded to the storage
+ * format and multiplied with the weights by 16-bit matrix instructions that accumulate in float32;
+ * bias added in float32, one rounding per output element.  (Layers that the LDS-halo kernel cannot
+ * serve are widened to float32 and computed there.)
+ * backward_*: the values are widened exactly, all products and sums are the float32 kernels', and
+ * each result element is rounded once, to nearest even.
+ * Same argument meaning and accumulate / overwrite contract as the _f32 calls (grad_input and
+ * grad_weight: rounded sum of their previous content and the gradient).  The workspace must come
+ * from dcn_workspace_bytes_for(2, ...): it also holds float copies of the tensors.  Offsets in 16
+ * bits limit the sampling positions to that format's grid (bfloat16: 1/128 voxel between 1 and 2,
+ * coarser above). */
 int dcn3d_forward_bf16(const void *input, const void *weight, const void *offset, const void *bias,
                        void *output, DCN3D_GEOMETRY, void *workspace, size_t workspace_bytes, void *stream);
 int dcn3d_backward_input_offset_bf16(const void *input, const void *weight, const void *offset,

@@ -1,8 +1,11 @@
 """16-bit storage entry points (dcn*_bf16, dcn*_f16) through the package's Functions: every tensor is
-stored as bfloat16 / binary16, the arithmetic is the float32 kernels' and each result is rounded
-once.  Oracle mode: the CPU oracle in float64 on the same 16-bit-rounded inputs.  A result then
-differs from the oracle by the float32 kernels' error plus one rounding to the storage format,
-half an ulp of the element: 2^-9 of its magnitude for bfloat16, 2^-12 for binary16.  Tolerances,
+stored as bfloat16 / binary16.  Backward: the tensors are widened exactly, the arithmetic is the
+float32 kernels' and each result is rounded once.  Forward: the columns are sampled in float32,
+rounded to the storage format and multiplied with the weights in 16-bit matrix instructions with
+float32 accumulation.  Oracle mode: the CPU oracle in float64 on the same 16-bit-rounded inputs.
+A gradient then differs from the oracle by the float32 kernels' error plus one rounding to the
+storage format, half an ulp of the element (2^-9 of its magnitude for bfloat16, 2^-12 for
+binary16); an output element additionally by the rounding of its sampled columns.  Tolerances,
 relative to the tensor's largest magnitude: bfloat16 5e-3, binary16 1e-3 forward / 2e-3 gradients.
 The reference has no such mode (deform3d/lib/deform_conv3d_cuda_kernel.cu:162-172 instantiates float only).
 """
@@ -54,16 +57,26 @@ def test_16bit_storage_medium_cases_match_oracle(name, dtype):
     _compare(make_case(*MEDIUM[name], dtype=dtype, seed=8), dtype, name)
 
 
-def test_16bit_results_are_the_float32_results_rounded_once():
-    """The bfloat16 output equals the float32 kernel's output on the widened inputs, rounded to bfloat16."""
+def test_16bit_gradients_are_the_float32_gradients_rounded_once():
+    """The backward entry points widen the tensors exactly, run the float32 kernels and round once: every
+    bfloat16 gradient element lies within one rounding (2^-8 of its magnitude; the float32 sums themselves
+    vary in their last bits with the order of the float atomics) of the float32 gradient on the widened
+    inputs.  (The forward pass multiplies in bfloat16 and is only close to the rounded float32 output.)"""
     import deform_conv3d_pytorch_op_amd as dcn
     c = make_case(*SMALL_CASES["3d_c4_like"], dtype=torch.bfloat16, seed=9)
     dev = torch.device("cuda:0")
-    x, off, w, b = (c[k].to(dev) for k in ("x", "off", "w", "b"))
     cfg = (c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
-    out16 = dcn.ConvOffset3dFunction.apply(x, off, w, b, *cfg)
-    out32 = dcn.ConvOffset3dFunction.apply(x.float(), off.float(), w.float(), b.float(), *cfg)
-    assert torch.equal(out16, out32.to(torch.bfloat16))
+    grads = {}
+    for dt in (torch.bfloat16, torch.float32):
+        x, off, w, b = (c[k].to(dev).to(dt).requires_grad_(True) for k in ("x", "off", "w", "b"))
+        out = dcn.ConvOffset3dFunction.apply(x, off, w, b, *cfg)
+        out.backward(c["gout"].to(dev).to(dt))
+        grads[dt] = (out.detach(), x.grad, off.grad, w.grad)
+    for g16, g32 in zip(grads[torch.bfloat16][1:], grads[torch.float32][1:]):
+        slack = 2.0 ** -8 * g32.abs() + 1e-6 * g32.abs().max()
+        assert bool(((g16.float() - g32).abs() <= slack).all())
+    out16, out32 = grads[torch.bfloat16][0].float(), grads[torch.float32][0]
+    assert (out16 - out32).abs().max().item() <= 5e-3 * out32.abs().max().item()
 
 
 def test_oob_zero_switch_is_float_only():

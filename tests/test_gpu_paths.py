@@ -44,6 +44,18 @@ SETTINGS = [
     {"DCN_OVERLAP_BACKWARD": "1", "DCN_FORWARD_SPLIT": "0"},
     {"DCN_FUSED_PAIR": "0", "DCN_FUSED_BREG2": "0"},
 ]
+MIXED_SETTINGS = [{"DCN_NATIVE16": "0"}]          # the 16-bit forward through the float32 kernels
+
+
+@pytest.mark.parametrize("extra", MIXED_SETTINGS, ids=lambda e: ",".join("%s=%s" % kv for kv in e.items()))
+def test_16bit_cases_under_knob(extra):
+    print("knobs", extra, flush=True)
+    env = dict(os.environ)
+    env.update(extra)
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.join(ROOT, "tests", "test_gpu_mixed.py"), "-q", "-x",
+                        "-m", "gpu", "--timeout", "120", "--timeout-method", "thread"],
+                       cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:]
 
 
 @pytest.mark.parametrize("extra", SETTINGS, ids=lambda e: ",".join("%s=%s" % kv for kv in e.items()))
