@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import dcn_oracle as orc
-from tests.cases import SMALL_CASES, make_case
+from tests.cases import SMALL_CASES, make_case, random_spec
 from tests.test_gpu_parity import rel_err, run_gpu
 
 pytestmark = pytest.mark.gpu
@@ -55,6 +55,15 @@ def test_16bit_storage_small_cases_match_oracle(name, dtype):
 def test_16bit_storage_medium_cases_match_oracle(name, dtype):
     print("16-bit case", name, dtype, flush=True)
     _compare(make_case(*MEDIUM[name], dtype=dtype, seed=8), dtype, name)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_16bit_storage_random_geometries_match_oracle(seed):
+    """Seeded random small (even seeds) and medium (odd seeds) geometries in both 16-bit formats."""
+    spec = random_spec(seed, medium=bool(seed % 2))
+    print("16-bit random geometry", seed, spec, flush=True)
+    for dtype in (torch.bfloat16, torch.float16):
+        _compare(make_case(*spec, dtype=dtype, seed=300 + seed), dtype, "random16_%d" % seed)
 
 
 def test_16bit_gradients_are_the_float32_gradients_rounded_once():
