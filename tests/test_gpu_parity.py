@@ -561,3 +561,34 @@ def test_error_paths_on_gpu_tensors():
         dcn.ConvOffset2dFunction.apply(x, torch.zeros(1, 18, 5, 6, device=dev), w, None, (1, 1), (1, 1), (1, 1), 4, 1)
     with pytest.raises(RuntimeError, match="input c != kernel c"):
         dcn.ConvOffset2dFunction.apply(x, torch.zeros(1, 18, 6, 6, device=dev), w, None, (1, 1), (1, 1), (1, 1), 4, 2)
+
+
+def test_every_sample_of_a_block_lands_in_one_cell():
+    """The worst case for the paired fixed-point LDS cells of the float32 fused backward kernel: the
+    offsets send all 27 taps of all 256 positions of a position block to the same voxel (integer
+    coordinates, so one corner carries the whole weight), and grad_output is parallel to every
+    weight column, which makes the Cauchy-Schwarz bound on the grad-column values an equality.
+    That cell then receives (positions x taps) terms, each at the bound the scale was chosen for."""
+    N, C, M, size = 1, 8, 16, (4, 8, 8)
+    g = torch.Generator().manual_seed(5)
+    v = torch.randn(M, generator=g, dtype=torch.float64)
+    w = v.view(M, 1, 1, 1, 1).expand(M, C, 3, 3, 3).contiguous()           # every (channel, tap) column is v
+    gout = v.view(1, M, 1, 1, 1).expand(N, M, *size).contiguous()           # every position's grad_output is v
+    x = torch.randn((N, C) + size, generator=g, dtype=torch.float64)
+    target = (1.0, 2.0, 3.0)
+    off = torch.zeros(N, 27, 3, *size, dtype=torch.float64)                 # one deformable group
+    for tap in range(27):
+        k = (tap // 9, (tap // 3) % 3, tap % 3)
+        for a in range(3):
+            pos = torch.arange(size[a], dtype=torch.float64).view([-1 if b == a else 1 for b in range(3)])
+            off[:, tap, a] = target[a] - (pos - 1 + k[a])                   # stride 1, pad 1, dilation 1
+    off = off.view(N, 81, *size)
+    c = dict(x=x.float(), off=off.float(), w=w.float(), b=None, gout=gout.float(), stride=(1, 1, 1), pad=(1, 1, 1),
+             dil=(1, 1, 1), cpg=C, groups=1, ins=size, k=(3, 3, 3), outs=size, nd=3)
+    got, want = run_gpu(c), run_oracle(c)
+    hit = want[1][0, :, 1, 2, 3]
+    assert float(hit.abs().min()) > 0.9 * 256 * 27 * float(v.dot(v))        # all terms arrived in that voxel
+    for name, a, b in zip(("output", "grad_input", "grad_offset", "grad_weight"), got, want):
+        tol = 1e-4 if name == "output" else 1e-3
+        e = rel_err(a, b)
+        assert e <= tol, "%s: relative error %.3e" % (name, e)
