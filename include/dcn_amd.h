@@ -102,7 +102,8 @@ int dcn3d_backward_input_offset_f64(const double *input, const double *weight, c
 /* Forward pass that allocates nothing and takes no workspace.  No counterpart in the reference: it
  * is for callers that cannot allocate device memory around the call (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  Same arguments, results and kernels as
- * dcn3d_forward_f32 without the workspace pair; the re-laid-out weight goes into a fixed device array
+ * dcn3d_forward_f32 without the workspace pair; the re-laid-out weight (and, for a layer of few
+ * positions, as many partial outputs as still fit) goes into a fixed device array
  * of DCN_NOALLOC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until
  * the process ends.  A layer whose re-laid-out weight is larger (roughly: 4 * kernel volume *
  * output_c rounded up to 256 * (input_c / group + 4) bytes) is rejected with DCN_E_WORKSPACE.  All
