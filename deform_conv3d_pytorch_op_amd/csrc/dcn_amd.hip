@@ -175,7 +175,10 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 // Halo tiling plan: block of output positions per workgroup, halo extents, channels per LDS pass.
 // Returns false when the geometry does not suit (halo too large for the staging table or LDS).
 // Tuning knobs (environment, read once per process):
-//   DCN_HALO_MARGIN        voxels of halo beyond the integer tap span on each side (default 2)
+//   DCN_HALO_MARGIN        voxels of halo beyond the integer tap span on each side: one fixed margin instead of
+//                          the choice on the device among 2, 3, 4 (3-D) or 2, 4, 6 (2-D)
+//   DCN_ADAPTIVE_MARGIN=0  always the smallest of those margins (2)
+//   DCN_TRACE_PLANS=1      print the halo plans and launches of every call on stderr
 //   DCN_LDS_BUDGET_KB      LDS per 512-thread workgroup of the forward halo kernel (default 72: two per CU)
 //   DCN_FORWARD_WG=512     never use the 1024-thread forward variant; =1024 use it whenever its halo fits
 //   DCN_FORWARD_SPLIT=n    forward pass: split the input channels of a position block over at most n workgroups (0: never)
@@ -281,28 +284,46 @@ static bool scatter_in_lds() {
     return v != 0;
 }
 #define LDS_BUDGET lds_budget()
-static int halo_margin() {      // DCN_HALO_MARGIN overrides the default of 2 voxels
+static int halo_margin() {      // DCN_HALO_MARGIN: one fixed margin; -1 when not set
     static const int v = [] {
         const char* e = getenv("DCN_HALO_MARGIN");
-        const int m = e ? atoi(e) : 2;
+        if (!e) return -1;
+        const int m = atoi(e);
         return m < 0 ? 0 : m;
     }();
     return v;
 }
+// Halo margins to plan for, ascending; the first is the one taken when nothing can be chosen.
+static int plan_margins(int nd, int* m) {
+    static const int adaptive = [] { const char* e = getenv("DCN_ADAPTIVE_MARGIN"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    if (halo_margin() >= 0) { m[0] = halo_margin(); return 1; }
+    m[0] = 2;
+    if (!adaptive) return 1;
+    m[1] = nd == 3 ? 3 : 4;
+    m[2] = nd == 3 ? 4 : 6;
+    return MAX_PLANS;
+}
+static_assert(MAX_PLANS == 3, "plan_margins fills three margins");
+static bool trace_plans() {             // DCN_TRACE_PLANS=1: the halo plans and launches of every call on stderr
+    static const int v = [] { const char* e = getenv("DCN_TRACE_PLANS"); return (e && atoi(e) != 0) ? 1 : 0; }();
+    return v != 0;
+}
+static int default_margin() { return halo_margin() >= 0 ? halo_margin() : 2; }
 static int forced_csplit() {    // DCN_CSPLIT=n: workgroups per (tile, deformable group) of the fused backward kernel
     static const int v = [] { const char* e = getenv("DCN_CSPLIT"); return e && atoi(e) > 0 ? atoi(e) : 0; }();
     return v;
 }
 
 template <typename T, int ND>
-bool plan_halo(Params& P, size_t budget, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH,
-               bool smallest_halo = false, int chunk_mult = 0) {
+bool plan_halo(Params& P, size_t budget, int m, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH,
+               bool smallest_halo = false, int chunk_mult = 0, const int* blocks = nullptr) {
     const int npos = waves * Mma<T>::TN;        // positions per workgroup, one column tile per wavefront
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
     else         { td[2] = 16; td[1] = npos / 16; }
-    const int m = halo_margin();
-    if (smallest_halo) {
+    if (blocks) {                               // the block shape of another plan
+        for (int a = 0; a < 3; ++a) td[a] = blocks[a];
+    } else if (smallest_halo) {
         // the block shape (powers of two, at least 4 positions along the fastest axis) with the
         // smallest halo: strided geometries want blocks that are short along the strided axes
         long long best = -1;
@@ -382,6 +403,18 @@ long long resident_workgroups(const void* kern, int threads, size_t lds) {
     return (long long)per_cu * cu_count();
 }
 
+static HaloPlan halo_plan_of(const Params& P) {
+    HaloPlan h;
+    for (int a = 0; a < 3; ++a) { h.hext[a] = P.hext[a]; h.mlo[a] = P.mlo[a]; }
+    h.hvol = P.hvol; h.hstride = P.hstride; h.cchunk = P.cchunk;
+    return h;
+}
+static bool same_blocks(const Params& a, const Params& b) {
+    for (int x = 0; x < 3; ++x)
+        if (a.tdim[x] != b.tdim[x] || a.ntile[x] != b.ntile[x]) return false;
+    return a.tiles == b.tiles;
+}
+
 template <typename K, typename... Args>
 int launch_halo(K kern, const char* name, dim3 grid, int threads, size_t lds, hipStream_t s, Args... args) {
     if (lds > 48 * 1024)
@@ -418,7 +451,7 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                                      forward_slab_elems<T>(P.kV, (mtiles_all + 7) / 8 * 8 * TN) * sizeof(T));
     {
         Params Pt = P;
-        const bool tiled = plan_halo<T, ND>(Pt, 144 * 1024, 1 << 30, sizeof(T), WAVESH, false, FQ);
+        const bool tiled = plan_halo<T, ND>(Pt, 144 * 1024, default_margin(), 1 << 30, sizeof(T), WAVESH, false, FQ);
         const long long tiles = tiled ? (long long)Pt.N * Pt.tiles : (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN));
         // (eight row tiles per wavefront only pay when the grid is full anyway: measured slower than
         // four with twice the sampling)
@@ -441,14 +474,15 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
     // Halo kernel: four channels of a voxel side by side in LDS (forward_quad_kernel).  Few
     // accumulators (MT <= 2): one 1024-thread workgroup per CU with the whole LDS, if its larger halo
     // fits and leaves 8 channels per pass.  Otherwise 512 threads: two workgroups per CU when that
-    // still leaves 8 channels per LDS pass, else one large one.
-    {
-        Params Ph = P;
+    // still leaves 8 channels per LDS pass, else one large one.  Returns the wavefronts per
+    // workgroup, 0 when no halo of margin m fits.
+    auto plan_for = [&](int m, Params& Ph) {
+        Ph = P;
         int nw = 0;
         // (the 3-D double instance of the 1024-thread shape does not fit its 128 registers)
         if (MT <= 2 && wide_forward() && !(sizeof(T) == 8 && ND == 3)) {
             Params Pw = P;
-            if (plan_halo<T, ND>(Pw, 144 * 1024, 1 << 30, sizeof(T), 16, false, FQ) &&
+            if (plan_halo<T, ND>(Pw, 144 * 1024, m, 1 << 30, sizeof(T), 16, false, FQ) &&
                 (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks <= 0x7fffffffLL &&
                 (wide_forward() == 2 || (Pw.cchunk >= 8 && (long long)Pw.N * Pw.tiles * Pw.G * Pw.mchunks >= cu_count()))) {
                 Ph = Pw;
@@ -456,24 +490,31 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
             }
         }
         if (!nw) {
-            bool tiled = plan_halo<T, ND>(Ph, LDS_BUDGET, 1 << 30, sizeof(T), WAVESH, false, FQ);
+            bool tiled = plan_halo<T, ND>(Ph, LDS_BUDGET, m, 1 << 30, sizeof(T), WAVESH, false, FQ);
             if ((!tiled || Ph.cchunk < 8) && LDS_BUDGET < 144 * 1024)
-                tiled = plan_halo<T, ND>(Ph, 144 * 1024, 1 << 30, sizeof(T), WAVESH, false, FQ) || tiled;
+                tiled = plan_halo<T, ND>(Ph, 144 * 1024, m, 1 << 30, sizeof(T), WAVESH, false, FQ) || tiled;
             if (!tiled || Ph.cchunk < 8) {       // strided layers: the block shape with the smallest halo may hold 8 channels
                 Params Ps = P;
-                if (plan_halo<T, ND>(Ps, 144 * 1024, 1 << 30, sizeof(T), WAVESH, true, FQ) && (!tiled || Ps.cchunk > Ph.cchunk)) {
+                if (plan_halo<T, ND>(Ps, 144 * 1024, m, 1 << 30, sizeof(T), WAVESH, true, FQ) && (!tiled || Ps.cchunk > Ph.cchunk)) {
                     Ph = Ps;
                     tiled = true;
                 }
             }
             if (tiled && (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks <= 0x7fffffffLL) nw = WAVESH;
         }
+        return nw;
+    };
+    {
+        int margins[MAX_PLANS];
+        const int nmargins = plan_margins(ND, margins);
+        Params plans[MAX_PLANS];
+        const int nw = plan_for(margins[0], plans[0]);
         const size_t slabs = (size_t)chunk_slot<FQ>(P.cpg, P.Cg, P.C_in - 1) + 1;
         const size_t wq_bytes = slabs * forward_slab_elems<T>(P.kV, P.Mp) * sizeof(S);
         if (nw == 16 || ws_bytes < align256(wq_bytes) + (size_t)fsplit * out_bytes) fsplit = 1;
         if (nw && ws_bytes >= wq_bytes) {
-            if (fsplit > 1) {
-                // channels per LDS pass such that every workgroup of a block gets the same number of passes
+            // channels per LDS pass such that every workgroup of a block gets the same number of passes
+            auto even_passes = [&](Params& Ph) {
                 auto chunks_of_group0 = [&](int cc) {
                     int n = 0;
                     for (int dg = 0; dg <= (P.Cg - 1) / P.cpg; ++dg) {
@@ -484,28 +525,79 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                 };
                 for (int cc = Ph.cchunk; cc >= FQ; cc -= FQ)
                     if (chunks_of_group0(cc) % fsplit == 0) { Ph.cchunk = cc; break; }
+            };
+            if (fsplit > 1) even_passes(plans[0]);
+            // Wider halos that one launch of the same kernel can serve as well (same workgroup shape and
+            // position blocks); the choice among them is made on the device, see PlanChoice.  The
+            // chosen index lives in the last 256 bytes of the workspace.
+            PlanChoice pc = {};
+            pc.nplans = 1;
+            pc.nd = ND;
+            pc.margin[0] = margins[0];
+            pc.base[0] = 1.f;
+            pc.far_wave = 1.5f;             // a wavefront with a sample beyond the halo gathers every channel of the pass from global memory
+            const size_t used = align256(wq_bytes) + (fsplit > 1 ? (size_t)fsplit * out_bytes : 0);
+            if (nmargins > 1 && ws_bytes >= used + 512) {
+                // (within the LDS of the first plan, which fixes how many workgroups share a CU; all of it
+                // when the grid gives a CU one workgroup at most)
+                const long long wgs = (long long)plans[0].N * plans[0].tiles * plans[0].G * plans[0].mchunks * fsplit;
+                size_t lds0 = (size_t)plans[0].cchunk * plans[0].hstride * sizeof(T) + (size_t)plans[0].hvol * 4;
+                if (wgs <= cu_count() && lds0 < 144 * 1024) lds0 = 144 * 1024;
+                for (int k = 1; k < nmargins; ++k) {
+                    Params& Pk = plans[pc.nplans];
+                    Pk = P;
+                    if (!plan_halo<T, ND>(Pk, lds0, margins[k], 1 << 30, sizeof(T), nw, false, FQ, plans[0].tdim)) continue;
+                    if (!same_blocks(Pk, plans[0]) || Pk.hvol > 3 * plans[0].hvol) continue;
+                    if (fsplit > 1) even_passes(Pk);
+                    pc.margin[pc.nplans] = margins[k];
+                    // staging and the per-pass geometry grow with the halo: about half of the kernel's time in 3-D, an eighth in 2-D
+                    pc.base[pc.nplans] = 1.f + (ND == 3 ? 0.5f : 0.12f) * ((float)Pk.hvol / (float)plans[0].hvol - 1.f);
+                    ++pc.nplans;
+                }
+                if (pc.nplans > 1) pc.sel = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + (ws_bytes - 256) / 256 * 256);
             }
+            for (int k = pc.nplans; k < MAX_PLANS; ++k) {
+                plans[k] = plans[0];
+                pc.margin[k] = pc.margin[pc.nplans - 1];
+                pc.base[k] = 1e30f;
+            }
+            PlanSet alts;
+            for (int k = 1; k < MAX_PLANS; ++k) alts.alt[k - 1] = halo_plan_of(plans[k]);
+            alts.mask = (1u << pc.nplans) - 1;
             {
                 const size_t total = (size_t)chunk_candidates<FQ>(P.cpg, P.Cg, P.C_in) * forward_slab_elems<T>(P.kV, P.Mp);
                 const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
-                hipLaunchKernelGGL((pack_forward_weight_kernel<T, S>), dim3(blocks), dim3(256), 0, s, Ph, w, wt);
+                const size_t n_off = (size_t)P.N * P.DG * P.kV * ND * P.outV;
+                hipLaunchKernelGGL((pack_forward_weight_kernel<T, S>), dim3(blocks + (pc.sel ? 1 : 0)), dim3(256), 0, s, plans[0], w, wt, pc, off, n_off);
                 if (int rc = check_launch("pack_forward_weight_kernel")) return rc;
             }
-            const size_t lds = (size_t)Ph.cchunk * Ph.hstride * sizeof(T) + (size_t)Ph.hvol * 4;
+            size_t lds = 0;
+            for (int k = 0; k < pc.nplans; ++k) {
+                const size_t l = (size_t)plans[k].cchunk * plans[k].hstride * sizeof(T) + (size_t)plans[k].hvol * 4;
+                if (l > lds) lds = l;
+            }
+            const Params& Ph = plans[0];
             const dim3 grid((unsigned)Ph.N * Ph.tiles * Ph.G * Ph.mchunks * fsplit);
+            if (trace_plans()) {
+                fprintf(stderr, "dcn forward: %d wavefronts, MT %d, grid %u, LDS %zu, split %d\n", nw, MT, grid.x, lds, fsplit);
+                for (int k = 0; k < pc.nplans; ++k)
+                    fprintf(stderr, "  plan %d: margin %d, halo %d x %d x %d, %d channels per pass, base cost %.3f\n", k, pc.margin[k],
+                            plans[k].hext[0], plans[k].hext[1], plans[k].hext[2], plans[k].cchunk, pc.base[k]);
+            }
             S* part = reinterpret_cast<S*>(static_cast<char*>(ws) + align256(wq_bytes));
             S* dst = fsplit > 1 ? part : out;
             const S* kbias = fsplit > 1 ? nullptr : bias;
+            const unsigned* sel = pc.sel;
             int rc;
             if (nw == 16) {
-                rc = MT == 1 ? launch_halo(forward_quad_kernel<T, ND, 1, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit)
-                             : launch_halo(forward_quad_kernel<T, ND, 2, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, in, off, wt, kbias, dst, fsplit);
+                rc = MT == 1 ? launch_halo(forward_quad_kernel<T, ND, 1, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit)
+                             : launch_halo(forward_quad_kernel<T, ND, 2, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit);
             } else {
                 switch (MT) {
-                    case 1: rc = launch_halo(forward_quad_kernel<T, ND, 1, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
-                    case 2: rc = launch_halo(forward_quad_kernel<T, ND, 2, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
-                    case 4: rc = launch_halo(forward_quad_kernel<T, ND, 4, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
-                    default: rc = launch_halo(forward_quad_kernel<T, ND, 8, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, in, off, wt, kbias, dst, fsplit); break;
+                    case 1: rc = launch_halo(forward_quad_kernel<T, ND, 1, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
+                    case 2: rc = launch_halo(forward_quad_kernel<T, ND, 2, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
+                    case 4: rc = launch_halo(forward_quad_kernel<T, ND, 4, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
+                    default: rc = launch_halo(forward_quad_kernel<T, ND, 8, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
                 }
             }
             if (rc || fsplit == 1) return rc;
@@ -582,121 +674,218 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     // Eight wavefronts per workgroup; four (half the positions, in the block shape with the smallest
     // halo) where only that fits, e.g. under stride 2.
     constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
+    using Kern = void (*)(Params, PlanSet, const unsigned*, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
+    struct FusedPlan {
+        Params Ph;
+        Kern kern;
+        int nw, cch, csplit, goff_atomic;
+        bool wide;
+        long long whole, items, slots;
+        size_t lds;
+        const T* wt;
+    };
+    const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;
+    // Plans the fused kernel for a halo of margin m; false when none of its shapes fits.
     // (attempts: eight wavefronts on the default block, eight on the block shape with the smallest
     // halo, four on the block shape with the smallest halo)
-    for (int attempt = fused_first_waves() == 8 ? 0 : 2; attempt < 3 && scatter_in_lds() && fused_coord(); ++attempt) {
-        const int nw = attempt < 2 ? 8 : 4;
-        const bool smallest = attempt > 0;
-        Params Ph = P;
-        // float32: two channels per LDS cell as 32-bit fixed point while the terms one cell can receive
-        // (positions of the block x taps) leave at least 17 bits below the largest possible term
-        const bool pair = sizeof(T) == 4 && fused_pair() && (long long)nw * TN * P.kV <= (1 << 14);
-        const size_t chb = (pair ? 4 : 8) + sizeof(T);      // LDS bytes per channel and halo voxel: cell + input value
-        if (!plan_halo<T, ND>(Ph, scatter_budget(), 8, chb, nw, smallest)) continue;
-        const size_t tables = (size_t)Ph.hvol * 4;      // halo table
-        const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * chb + tables <= scatter_budget();
-        if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
-        if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) < 4) continue;
-        // Channels per chunk: 8 where that takes fewer MFMA passes per channel (a pass holds TN / CCH
-        // taps: the 9 taps of a 3x3 kernel are 2 float passes per 4 channels or 3 per 8; the 27 of a
-        // 3x3x3 kernel 4 or 7) and the planes of 8 channels fit: the small halos of 2-D layers, and
-        // 3-D ones with paired cells.
-        const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;
-        auto passes = [&](int c) { const int tp = Mma<T>::TN / c; return (P.kV + tp - 1) / tp; };
-        const bool eight = (ND == 2 || pair) && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
-                           (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 8;
-        const int cch = eight ? 8 : 4;
-        Ph.cchunk = cch;
-        if (fixed && !eight) Ph.hstride = FUSED_HS;
-        const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
-        // grad_output operand held in registers when its reduction steps fit: 32 per pass
-        // (M <= 64 float, 128 double with 4-channel chunks)
-        const int ksteps = (P.M + Mma<T>::KL - 1) / Mma<T>::KL;
-        const bool wide = eight && pair && ksteps <= 32;                                         // the kernel's WIDE
-        const int slot_regs = wide ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
-        const bool breg = ksteps <= Mma<T>::NACC / slot_regs * (wide ? 16 : 8);
-        // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
-        const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
-        {   // weights in the lane order of the kernel's operand loads, one slab per channel chunk
+    auto plan_fused = [&](int m, FusedPlan& fp) {
+        for (int attempt = fused_first_waves() == 8 ? 0 : 2; attempt < 3; ++attempt) {
+            const int nw = attempt < 2 ? 8 : 4;
+            const bool smallest = attempt > 0;
+            Params Ph = P;
+            // float32: two channels per LDS cell as 32-bit fixed point while the terms one cell can receive
+            // (positions of the block x taps) leave at least 17 bits below the largest possible term
+            const bool pair = sizeof(T) == 4 && fused_pair() && (long long)nw * TN * P.kV <= (1 << 14);
+            const size_t chb = (pair ? 4 : 8) + sizeof(T);      // LDS bytes per channel and halo voxel: cell + input value
+            if (!plan_halo<T, ND>(Ph, scatter_budget(), m, 8, chb, nw, smallest)) continue;
+            const size_t tables = (size_t)Ph.hvol * 4;      // halo table
+            const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * chb + tables <= scatter_budget();
+            if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
+            if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) < 4) continue;
+            // Channels per chunk: 8 where that takes fewer MFMA passes per channel (a pass holds TN / CCH
+            // taps: the 9 taps of a 3x3 kernel are 2 float passes per 4 channels or 3 per 8; the 27 of a
+            // 3x3x3 kernel 4 or 7) and the planes of 8 channels fit: the small halos of 2-D layers, and
+            // 3-D ones with paired cells.
+            auto passes = [&](int c) { const int tp = Mma<T>::TN / c; return (P.kV + tp - 1) / tp; };
+            const bool eight = (ND == 2 || pair) && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
+                               (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 8;
+            const int cch = eight ? 8 : 4;
+            Ph.cchunk = cch;
+            if (fixed && !eight) Ph.hstride = FUSED_HS;
+            const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
+            // grad_output operand held in registers when its reduction steps fit: 32 per pass
+            // (M <= 64 float, 128 double with 4-channel chunks)
+            const int ksteps = (P.M + Mma<T>::KL - 1) / Mma<T>::KL;
+            const bool wide = eight && pair && ksteps <= 32;                                         // the kernel's WIDE
+            const int slot_regs = wide ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
+            const bool breg = ksteps <= Mma<T>::NACC / slot_regs * (wide ? 16 : 8);
+            // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
+            const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
+            Kern kern = nullptr;
+#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>
+#define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2>
+            auto pick = [&](auto pair_tag) {
+                constexpr bool PR = decltype(pair_tag)::value;
+                if (eight) {
+                    if constexpr (ND == 2 || PR) kern = breg ? DCN_FUSED_C(8, true, 0, 8, PR) : DCN_FUSED_C(8, false, 0, 8, PR);
+                } else if (breg2) {
+                    if constexpr (sizeof(T) == 4) {
+                        if (nw == 8) kern = fixed ? DCN_FUSED_B2(FUSED_HS, 8, PR) : DCN_FUSED_B2(0, 8, PR);
+                        else kern = fixed ? DCN_FUSED_B2(FUSED_HS, 4, PR) : DCN_FUSED_B2(0, 4, PR);
+                    }
+                } else if (nw == 8)
+                    kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 8, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 8, PR) : DCN_FUSED_C(4, false, 0, 8, PR);
+                else
+                    kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 4, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 4, PR) : DCN_FUSED_C(4, false, 0, 4, PR);
+            };
+            if constexpr (sizeof(T) == 4) {
+                if (pair) pick(std::true_type{});
+                else pick(std::false_type{});
+            } else
+                pick(std::false_type{});
+#undef DCN_FUSED_B2
+#undef DCN_FUSED_C
+            if (!kern) continue;
+            // Work items are (tile, deformable group) pairs, each a run of nchunks channel chunks.  `slots`
+            // workgroups run at once, so the items take whole rounds plus a partly filled last one.  Either
+            // every item is split over 1, 2 or 4 workgroups (workgroup cz takes every csplit-th chunk), or
+            // the items of the whole rounds stay unsplit and only those of the last round are split, as
+            // finely as fills the device; they come last in the launch.  A workgroup's fixed part
+            // (grad_output operand, halo table, offsets) costs about a quarter of a chunk, which the
+            // estimate charges per split.  The chunks of an item add their grad_offset parts with float
+            // atomics on a zero-filled buffer (measured faster than read-modify-write by one workgroup);
+            // an item of a single chunk stores.
+            const int nchunks = (seg + cch - 1) / cch;
+            const long long items = (long long)Ph.N * Ph.tiles * Ph.DG;
+            const long long slots = forced_slots() ? forced_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
+            auto item_cost = [&](double chunks_per_wg, int wgs) { return wgs * (chunks_per_wg + 0.25) / nchunks; };
+            int csplit = 1;
+            long long whole = 0;                              // unsplit items at the start of the launch
+            double best = 1e30;
+            for (int cs = 1; cs <= 4 && cs <= nchunks; cs *= 2) {
+                const double rounds = (double)((items * cs + slots - 1) / slots) / cs * item_cost((double)nchunks / cs, cs);
+                if (rounds < best) { best = rounds; csplit = cs; }
+            }
+            if (fused_tail_split() && items > slots && items % slots) {
+                const long long rest = items % slots;
+                const long long cs = slots / rest < nchunks ? slots / rest : nchunks;
+                if (cs >= 2) {
+                    const double rounds = (double)(items / slots) * item_cost(nchunks, 1) + item_cost((double)((nchunks + cs - 1) / cs), 1);
+                    if (rounds < best) { best = rounds; csplit = (int)cs; whole = items - rest; }
+                }
+            }
+            if (forced_csplit()) { csplit = forced_csplit(); whole = 0; }
+            if (csplit > nchunks) csplit = nchunks;
+            if (whole + (items - whole) * csplit > 0x7fffffffLL) continue;
+            fp.Ph = Ph; fp.kern = kern; fp.nw = nw; fp.cch = cch; fp.csplit = csplit; fp.goff_atomic = nchunks > 1 ? 1 : 0;
+            fp.wide = wide; fp.whole = whole; fp.items = items; fp.slots = slots; fp.lds = lds; fp.wt = nullptr;
+            return true;
+        }
+        return false;
+    };
+    FusedPlan fp[MAX_PLANS];
+    int margins[MAX_PLANS];
+    const int nmargins = plan_margins(ND, margins);
+    if (scatter_in_lds() && fused_coord() && plan_fused(margins[0], fp[0])) {
+        // Wider halos for offsets that reach further; the choice is made on the device, see
+        // PlanChoice.  A plan whose weights want another lane order gets a packed copy of its own in
+        // the region of the channels-last input, which this path does not use.
+        PlanChoice pc = {};
+        pc.nplans = 1;
+        pc.nd = ND;
+        pc.margin[0] = margins[0];
+        pc.base[0] = 1.f;
+        pc.far_sample = ND == 3 ? 4.5f : 1.f;       // a sample beyond the halo scatters with global atomics
+        int copies = 1;                             // packed weight copies
+        fp[0].wt = wt;
+        for (int k = 1; k < nmargins; ++k) {
+            FusedPlan& c = fp[pc.nplans];
+            if (!plan_fused(margins[k], c) || c.nw != fp[0].nw || c.Ph.hvol > 3 * fp[0].Ph.hvol) continue;
+            for (int e = 0; e < pc.nplans && !c.wt; ++e)
+                if (fp[e].cch == c.cch && fp[e].wide == c.wide) c.wt = fp[e].wt;
+            if (!c.wt) {
+                if ((size_t)copies * wbytes > tbytes) continue;
+                c.wt = reinterpret_cast<const T*>(reinterpret_cast<const char*>(in_cl) + (size_t)(copies - 1) * wbytes);
+                ++copies;
+            }
+            pc.margin[pc.nplans] = margins[k];
+            // flush, staging and the per-chunk passes grow with the halo: most of the kernel's time in 3-D, little in 2-D
+            pc.base[pc.nplans] = 1.f + (ND == 3 ? 0.9f : 0.05f) * ((float)c.Ph.hvol / (float)fp[0].Ph.hvol - 1.f);
+            ++pc.nplans;
+        }
+        for (int k = pc.nplans; k < MAX_PLANS; ++k) {
+            pc.margin[k] = pc.margin[pc.nplans - 1];
+            pc.base[k] = 1e30f;
+        }
+        unsigned* sel = pc.nplans > 1 ? reinterpret_cast<unsigned*>(wmax + 16) : nullptr;
+        pc.sel = sel;
+        const size_t n_off = (size_t)P.N * P.DG * P.kV * ND * P.outV;
+        // weights in the lane order of the kernel's operand loads, one slab per channel chunk; the
+        // first launch clears the weight bounds and chooses the plan
+        for (int k = 0; k < pc.nplans; ++k) {
+            bool packed = false;
+            for (int e = 0; e < k; ++e) packed = packed || fp[e].wt == fp[k].wt;
+            if (packed) continue;
+            const bool eight = fp[k].cch == 8, wide = fp[k].wide;
             const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)(eight ? chunk_candidates<8>(P.cpg, P.Cg, P.C_in)
-                                                                                      : chunk_candidates<4>(P.cpg, P.Cg, P.C_in)), cch);
+                                                                                      : chunk_candidates<4>(P.cpg, P.Cg, P.C_in)), fp[k].cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
+            PlanChoice pk = pc;
+            if (k > 0) pk.sel = nullptr;
+            float* bounds = k == 0 ? wmax : nullptr;
+            T* dst = const_cast<T*>(fp[k].wt);
+            const dim3 pgrid(blocks + (pk.sel ? 1 : 0));
             // (wide: row order that leaves the eight channels of a tap in one lane)
-            if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);
-            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);
-            else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), dim3(blocks), dim3(256), 0, s, P, w, wt, wmax);
+            if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
         if (int rc = weight_bounds<T>(P, w, wmax, s)) return rc;
-        using Kern = void (*)(Params, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
-        Kern kern = nullptr;
-#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>
-#define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2>
-        auto pick = [&](auto pair_tag) {
-            constexpr bool PR = decltype(pair_tag)::value;
-            if (eight) {
-                if constexpr (ND == 2 || PR) kern = breg ? DCN_FUSED_C(8, true, 0, 8, PR) : DCN_FUSED_C(8, false, 0, 8, PR);
-            } else if (breg2) {
-                if constexpr (sizeof(T) == 4) {
-                    if (nw == 8) kern = fixed ? DCN_FUSED_B2(FUSED_HS, 8, PR) : DCN_FUSED_B2(0, 8, PR);
-                    else kern = fixed ? DCN_FUSED_B2(FUSED_HS, 4, PR) : DCN_FUSED_B2(0, 4, PR);
-                }
-            } else if (nw == 8)
-                kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 8, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 8, PR) : DCN_FUSED_C(4, false, 0, 8, PR);
-            else
-                kern = fixed && breg ? DCN_FUSED_C(4, true, FUSED_HS, 4, PR) : fixed ? DCN_FUSED_C(4, false, FUSED_HS, 4, PR) : DCN_FUSED_C(4, false, 0, 4, PR);
-        };
-        if constexpr (sizeof(T) == 4) {
-            if (pair) pick(std::true_type{});
-            else pick(std::false_type{});
-        } else
-            pick(std::false_type{});
-#undef DCN_FUSED_B2
-#undef DCN_FUSED_C
-        if (!kern) continue;
-        if (lds > 48 * 1024)
-            if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return rc;
-        // Work items are (tile, deformable group) pairs, each a run of nchunks channel chunks.  `slots`
-        // workgroups run at once, so the items take whole rounds plus a partly filled last one.  Either
-        // every item is split over 1, 2 or 4 workgroups (workgroup cz takes every csplit-th chunk), or
-        // the items of the whole rounds stay unsplit and only those of the last round are split, as
-        // finely as fills the device; they come last in the launch.  A workgroup's fixed part
-        // (grad_output operand, halo table, offsets) costs about a quarter of a chunk, which the
-        // estimate charges per split.  The chunks of an item add their grad_offset parts with float
-        // atomics on a zero-filled buffer (measured faster than read-modify-write by one workgroup);
-        // an item of a single chunk stores.
-        const int nchunks = (seg + cch - 1) / cch;
-        const long long items = (long long)Ph.N * Ph.tiles * Ph.DG;
-        const long long slots = forced_slots() ? forced_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
-        auto item_cost = [&](double chunks_per_wg, int wgs) { return wgs * (chunks_per_wg + 0.25) / nchunks; };
-        int csplit = 1;
-        long long whole = 0;                              // unsplit items at the start of the launch
-        double best = 1e30;
-        for (int cs = 1; cs <= 4 && cs <= nchunks; cs *= 2) {
-            const double rounds = (double)((items * cs + slots - 1) / slots) / cs * item_cost((double)nchunks / cs, cs);
-            if (rounds < best) { best = rounds; csplit = cs; }
-        }
-        if (fused_tail_split() && items > slots && items % slots) {
-            const long long rest = items % slots;
-            const long long cs = slots / rest < nchunks ? slots / rest : nchunks;
-            if (cs >= 2) {
-                const double rounds = (double)(items / slots) * item_cost(nchunks, 1) + item_cost((double)((nchunks + cs - 1) / cs), 1);
-                if (rounds < best) { best = rounds; csplit = (int)cs; whole = items - rest; }
-            }
-        }
-        if (forced_csplit()) { csplit = forced_csplit(); whole = 0; }
-        if (csplit > nchunks) csplit = nchunks;
-        const int goff_atomic = nchunks > 1 ? 1 : 0;
-        if (goff_atomic) {
+        bool any_atomic = false;
+        for (int k = 0; k < pc.nplans; ++k) any_atomic = any_atomic || fp[k].goff_atomic;
+        if (any_atomic) {
             const size_t nel = (size_t)P.N * P.DG * P.kV * ND * P.outV;
             const unsigned fb = (unsigned)((nel + 1023) / 1024 > 8192 ? 8192 : (nel + 1023) / 1024);
             hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fb), dim3(256), 0, s, goff, nel);
             if (int rc = check_launch("fill_zero_kernel")) return rc;
         }
-        if (whole + (items - whole) * csplit > 0x7fffffffLL) return fail(DCN_E_ARGUMENT, "too many workgroups for one launch");
-        hipLaunchKernelGGL(kern, dim3((unsigned)(whole + (items - whole) * csplit)), dim3(nw * 64), lds, s, Ph, in, off, wt, gout,
-                           wmax, gin, goff, csplit, (unsigned)whole, goff_atomic);
-        if (int rc = check_launch("backward_input_halo_kernel")) return rc;
+        // one launch per set of plans that differ in nothing but the halo
+        unsigned launched = 0;
+        for (int k = 0; k < pc.nplans; ++k) {
+            if ((launched >> k) & 1u) continue;
+            // (the kernel takes plan 0 as its Params argument: a launch that does not serve plan 0 gets
+            // the Params of its first plan there, which its mask never selects as such)
+            PlanSet alts;
+            alts.mask = 0;
+            size_t lds = 0;
+            for (int e = 1; e < MAX_PLANS; ++e) alts.alt[e - 1] = halo_plan_of(fp[k].Ph);
+            for (int e = k; e < pc.nplans; ++e) {
+                const bool same = fp[e].kern == fp[k].kern && fp[e].wt == fp[k].wt && fp[e].csplit == fp[k].csplit && fp[e].whole == fp[k].whole &&
+                                  fp[e].items == fp[k].items && fp[e].goff_atomic == fp[k].goff_atomic && fp[e].nw == fp[k].nw &&
+                                  fp[e].slots == fp[k].slots && same_blocks(fp[e].Ph, fp[k].Ph);      // (as many workgroups per CU with the larger LDS)
+                if (!same) continue;
+                if (e > 0) alts.alt[e - 1] = halo_plan_of(fp[e].Ph);
+                alts.mask |= 1u << e;
+                if (fp[e].lds > lds) lds = fp[e].lds;
+            }
+            launched |= alts.mask;
+            if (trace_plans()) {
+                fprintf(stderr, "dcn backward_input_offset: launch for plans %#x: %d wavefronts, %d channels per chunk%s, grid %lld (%lld unsplit, rest x %d), LDS %zu\n",
+                        alts.mask, fp[k].nw, fp[k].cch, fp[k].wide ? " (wide)" : "", fp[k].whole + (fp[k].items - fp[k].whole) * fp[k].csplit, fp[k].whole,
+                        fp[k].csplit, lds);
+                for (int e = 0; e < pc.nplans; ++e)
+                    if ((alts.mask >> e) & 1u)
+                        fprintf(stderr, "  plan %d: margin %d, halo %d x %d x %d, base cost %.3f\n", e, pc.margin[e], fp[e].Ph.hext[0], fp[e].Ph.hext[1],
+                                fp[e].Ph.hext[2], pc.base[e]);
+            }
+            if (lds > 48 * 1024)
+                if (int rc = raise_lds_limit(reinterpret_cast<const void*>(fp[k].kern), lds)) return rc;
+            hipLaunchKernelGGL(fp[k].kern, dim3((unsigned)(fp[k].whole + (fp[k].items - fp[k].whole) * fp[k].csplit)), dim3(fp[k].nw * 64), lds, s,
+                               fp[k].Ph, alts, (const unsigned*)sel, in, off, fp[k].wt, gout, (const float*)wmax, gin, goff, fp[k].csplit, (unsigned)fp[k].whole,
+                               fp[k].goff_atomic);
+            if (int rc = check_launch("backward_input_halo_kernel")) return rc;
+        }
         return DCN_OK;
     }
 
@@ -710,7 +899,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
     if (int rc = check_launch("to_channels_last_kernel")) return rc;
     Params Ph = P;
-    bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), 8, 8);
+    bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), default_margin(), 8, 8);
     if (halo && (long long)Ph.N * Ph.tiles * Ph.DG > 0x7fffffffLL) halo = false;
     if (halo) {                                     // the scatter kernel packs 4 or 8 channels per MFMA tile
         const size_t fit = (scatter_budget() - (size_t)Ph.hvol * 4) / ((size_t)Ph.hstride * 8);
@@ -735,12 +924,16 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG);
         T* nogoff = nullptr;
+        PlanSet alts;
+        for (int e = 1; e < MAX_PLANS; ++e) alts.alt[e - 1] = halo_plan_of(Ph);
+        alts.mask = 1u;
+        const unsigned* nosel = nullptr;
         if (Ph.cchunk == 8)
             return launch_halo(backward_input_halo_kernel<T, ND, 8, false, false, 0, WAVESH>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
-                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1, 0u, 0);
+                               Ph, alts, nosel, in, off, (const T*)wt, gout, (const float*)wmax, gin, nogoff, 1, 0u, 0);
         if (Ph.cchunk == 4)
             return launch_halo(backward_input_halo_kernel<T, ND, 4, false, false, 0, WAVESH>, "backward_input_halo_kernel", hgrid, WGH, lds, s,
-                               Ph, in, off, wt, gout, wmax, gin, nogoff, 1, 0u, 0);
+                               Ph, alts, nosel, in, off, (const T*)wt, gout, (const float*)wmax, gin, nogoff, 1, 0u, 0);
         return fail(DCN_E_LAUNCH, "no scatter kernel for this channel chunk");
     }
     // halo does not fit in LDS: scatter with global atomics on the channels-last copy

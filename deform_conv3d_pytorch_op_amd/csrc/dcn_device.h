@@ -34,6 +34,52 @@ struct Params {
     int oob_zero;                 // 3-D backward: 1 = no grad_offset term for out-of-range samples
 };
 
+// Halo margin chosen on the device.  How far the LDS halo of a position block must reach depends on
+// the offsets, which the host never sees: a sample whose corners lie outside the halo takes a slow
+// path through global memory, and a halo wider than the offsets need costs LDS that the channels
+// could have used.  The host therefore plans the halo kernels for up to MAX_PLANS margins (same
+// position blocks, so the plans differ in the fields of HaloPlan only); one
+// block of the weight-packing kernel that precedes them counts, over a spread of the offsets, how
+// many reach past each margin, prices every plan and writes the index of the cheapest to *sel.  A
+// kernel launch serves the plans of its `mask` and returns at once when another one was chosen.
+constexpr int MAX_PLANS = 3;
+struct HaloPlan {                 // what a margin changes in Params
+    int hext[3], mlo[3], hvol, hstride, cchunk;
+};
+struct PlanSet {
+    HaloPlan alt[MAX_PLANS - 1];  // plans 1 .. MAX_PLANS - 1 (plan 0 is the Params argument itself)
+    unsigned mask;                // bit i: this launch runs plan i
+};
+struct PlanChoice {
+    unsigned* sel;                // chosen plan (device memory), null: a single plan, nothing to choose
+    int nplans, nd;
+    int margin[MAX_PLANS];        // ascending
+    float base[MAX_PLANS];        // cost of the plan when no sample leaves its halo, plan 0 = 1
+    // cost added by samples beyond the halo, as a factor 1 + far_wave * P(some lane of a wavefront
+    // holds such a sample) + far_sample * P(a sample is one)
+    float far_wave, far_sample;
+};
+// The halo fields of the chosen plan in H; false when this launch does not serve it (uniform for
+// the grid).  Kept apart from P, which stays the kernel argument: its other fields can then be
+// re-read from the argument segment wherever they are needed instead of living in registers.
+// (field by field from constant argument offsets, no indexed copy)
+__device__ inline bool chosen_halo(const Params& P, const PlanSet& S, const unsigned* __restrict__ sel, HaloPlan& H) {
+    unsigned idx = 0;
+    if (sel) idx = (unsigned)__builtin_amdgcn_readfirstlane((int)*sel);
+    if (idx >= (unsigned)MAX_PLANS || !((S.mask >> idx) & 1u)) return false;
+    static_assert(MAX_PLANS == 3, "two alternatives are selected between");
+    const bool zero = idx == 0, one = idx == 1;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        H.hext[a] = zero ? P.hext[a] : one ? S.alt[0].hext[a] : S.alt[1].hext[a];
+        H.mlo[a] = zero ? P.mlo[a] : one ? S.alt[0].mlo[a] : S.alt[1].mlo[a];
+    }
+    H.hvol = zero ? P.hvol : one ? S.alt[0].hvol : S.alt[1].hvol;
+    H.hstride = zero ? P.hstride : one ? S.alt[0].hstride : S.alt[1].hstride;
+    H.cchunk = zero ? P.cchunk : one ? S.alt[0].cchunk : S.alt[1].cchunk;
+    return true;
+}
+
 // ---------------------------------------------------------------------------------------------
 template <typename T> struct Mma;
 

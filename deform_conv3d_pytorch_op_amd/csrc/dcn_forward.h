@@ -62,14 +62,21 @@ __host__ __device__ inline size_t forward_slab_elems(int kV, int Mp) {
     return (size_t)((kV + Mma<T>::KL - 1) / Mma<T>::KL) * Mp * Mma<T>::KL * FQ;
 }
 
+// With pc.sel set the launch has one block more, which chooses the halo plan from the offsets.
 template <typename T, typename S = T>
-__global__ void pack_forward_weight_kernel(Params P, const S* __restrict__ W, S* __restrict__ Wq) {
+__global__ void pack_forward_weight_kernel(Params P, const S* __restrict__ W, S* __restrict__ Wq, PlanChoice pc,
+                                           const S* __restrict__ off, size_t n_off) {
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL;
+    const unsigned pack_blocks = pc.sel ? gridDim.x - 1 : gridDim.x;
+    if (blockIdx.x == pack_blocks) {
+        choose_plan(pc, off, n_off);
+        return;
+    }
     const int mtiles = P.Mp / TN;
     const size_t per_slab = forward_slab_elems<T>(P.kV, P.Mp);
     const size_t total = (size_t)chunk_candidates<FQ>(P.cpg, P.Cg, P.C_in) * per_slab;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)pack_blocks * blockDim.x) {
         const int c0 = chunk_candidate<FQ>(P.cpg, P.Cg, (int)(i / per_slab));       // candidate first channel of a group
         const int seg_b = max(c0 / P.cpg * P.cpg, c0 / P.Cg * P.Cg);
         if ((c0 - seg_b) % FQ) continue;
@@ -91,10 +98,10 @@ __global__ void pack_forward_weight_kernel(Params P, const S* __restrict__ W, S*
 // of a short last group and halo voxels outside the volume hold zero (a sample in the rim reads
 // the latter with weight zero).
 template <typename T, int WGS, typename S = T>
-__device__ inline void halo_stage_quads(const Params& P, const S* __restrict__ chan0, int nch,
+__device__ inline void halo_stage_quads(const Params& P, const HaloPlan& H, const S* __restrict__ chan0, int nch,
                                         const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
     const int ngrp = (nch + FQ - 1) / FQ;
-    for (int v = threadIdx.x; v < P.hvol; v += WGS) {
+    for (int v = threadIdx.x; v < H.hvol; v += WGS) {
         const unsigned t = sTab[v];
         const unsigned g = t == ~0u ? 0u : t;
         for (int grp = 0; grp < ngrp; ++grp) {
@@ -103,7 +110,7 @@ __device__ inline void halo_stage_quads(const Params& P, const S* __restrict__ c
             for (int e = 0; e < FQ; ++e) val[e] = Store<S>::ld(chan0[(size_t)min(grp * FQ + e, nch - 1) * P.inV + g]);
 #pragma unroll
             for (int e = 0; e < FQ; ++e)
-                sIn[((size_t)grp * P.hstride + v) * FQ + e] = (grp * FQ + e < nch && t != ~0u) ? val[e] : (T)0;
+                sIn[((size_t)grp * H.hstride + v) * FQ + e] = (grp * FQ + e < nch && t != ~0u) ? val[e] : (T)0;
         }
     }
 }
@@ -118,16 +125,19 @@ __device__ inline void halo_stage_quads(const Params& P, const S* __restrict__ c
 // shape, so that two of its workgroups share a CU)
 // S: storage format of the tensors (see Store); with a 16-bit format T is float and csplit must be 1.
 template <typename T, int ND, int MT, int NW, typename S = T>
-__global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, const S* __restrict__ in,
+__global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
+                                                           const S* __restrict__ in,
                                                            const S* __restrict__ off, const S* __restrict__ Wq,
                                                            const S* __restrict__ bias, S* __restrict__ out, int csplit) {
+    HaloPlan H;
+    if (!chosen_halo(P, alts, sel, H)) return;          // another launch runs the chosen plan
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, WGS = NW * 64;
     constexpr bool S16 = sizeof(S) == 2;                // 16-bit storage: 16-bit matrix instructions
     typedef T V4 __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sIn = reinterpret_cast<T*>(smem_raw);                                            // [cchunk / 4][hstride][4]
-    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)P.cchunk * P.hstride);   // [hvol]
+    unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)H.cchunk * H.hstride);   // [hvol]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     // workgroups of one tile are neighbours in an XCD-contiguous order
@@ -138,7 +148,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
 
     TileGeo<ND> tg_;
-    tile_decode<ND>(P, wg / (unsigned)(P.G * P.mchunks), tg_);
+    tile_decode<ND>(P, H, wg / (unsigned)(P.G * P.mchunks), tg_);
     const int n = tg_.n;
     int o[ND];
     unsigned pos;
@@ -148,7 +158,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     T ibf[ND];
 #pragma unroll
     for (int a = 0; a < ND; ++a) ibf[a] = (T)(o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)]);
-    halo_table<ND, WGS>(P, tg_, sTab);             // visible after the first barrier below
+    halo_table<ND, WGS>(P, H, tg_, sTab);             // visible after the first barrier below
 
     typename MM::Acc acc[MT];
 #pragma unroll
@@ -161,8 +171,8 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     unsigned coff[NC];
 #pragma unroll
     for (int i = 0; i < NC; ++i)
-        coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * P.hext[1] + ((i >> 1) & 1)) * P.hext[2] + (i & 1))
-                          : (unsigned)(((i >> 1) & 1) * P.hext[2] + (i & 1));
+        coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * H.hext[1] + ((i >> 1) & 1)) * H.hext[2] + (i & 1))
+                          : (unsigned)(((i >> 1) & 1) * H.hext[2] + (i & 1));
     // this lane's weights of (tap group 0, first row tile of the chunk) inside a slab
     const unsigned w_lane = (((unsigned)mchunk * MT * KL + q) * TN + j) * FQ;
     const unsigned w_tile = (unsigned)KL * TN * FQ;               // one row tile further
@@ -173,13 +183,13 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
         const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
         const S* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
-        for (int cc0 = cb; cc0 < ce; cc0 += P.cchunk) {
+        for (int cc0 = cb; cc0 < ce; cc0 += H.cchunk) {
             if ((chunk_no++) % csplit != cz) continue;                     // another workgroup's chunk (uniform)
-            const int nch = min(P.cchunk, ce - cc0);
+            const int nch = min(H.cchunk, ce - cc0);
             const int ngrp = (nch + FQ - 1) / FQ;
             const S* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
             __syncthreads();                                               // readers of the previous chunk are done
-            halo_stage_quads<T, WGS, S>(P, chan0, nch, sTab, sIn);
+            halo_stage_quads<T, WGS, S>(P, H, chan0, nch, sTab, sIn);
             __syncthreads();
             // slabs of consecutive groups of one segment are consecutive.  Uniform base (scalar
             // registers); the lanes add the 32-bit offset w_lane.
@@ -223,12 +233,12 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
                     f[a] = pc - fl;
                     inside = inside && fabs(pa - pc) < (T)1;                // -1 < p < size, false for NaN
                     u[a] = (int)fl - tg_.hb[a];
-                    inhalo = inhalo && (unsigned)u[a] < (unsigned)(P.hext[sa] - 1);
+                    inhalo = inhalo && (unsigned)u[a] < (unsigned)(H.hext[sa] - 1);
                 }
                 const bool near = inside && inhalo, far = inside && !inhalo;
                 unsigned base;
-                if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], P.hext[1]) + u[1], P.hext[2]) + u[2]);
-                else base = (unsigned)(__mul24(u[0], P.hext[2]) + u[1]);
+                if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], H.hext[1]) + u[1], H.hext[2]) + u[2]);
+                else base = (unsigned)(__mul24(u[0], H.hext[2]) + u[1]);
                 base = near ? base : 0u;           // lanes without a sample in the halo read cell 0 and drop the value
                 T cw[NC];                          // corner weights, w_l * w_h * w_w
                 if constexpr (ND == 3) {
@@ -304,7 +314,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
                             for (int mt = 0; mt < MT; ++mt) acc[mt] = MM::mma(a4[mt][e], b, acc[mt]);
                         }
                     }
-                    hp += P.hstride;
+                    hp += H.hstride;
                     wp += per_slab;
                 }
                 if (__any(far)) {                  // rare: some sample of this wave reaches past the halo

@@ -62,20 +62,89 @@ __host__ __device__ inline int chunk_candidate(int cpg, int Cg, int y) {     // 
     return y / cps * seg + y % cps * CCH;
 }
 
+// One block of 256 threads chooses the halo plan of the launches that follow (see PlanChoice).
+// It reads 32 runs of 256 consecutive offset entries spread evenly over the tensor (all of a small
+// one); an entry v keeps a sample inside a halo of margin m along its axis when -m <= v < m (the
+// low corner floor(v) is at least -m, the high corner floor(v) + 1 at most m).  From the fraction
+// e of entries beyond margin m: a sample leaves the halo with probability p = 1 - (1 - e)^nd, a
+// wavefront holds such a sample with probability 1 - (1 - p)^64.
+__device__ inline float offset_value(float v) { return v; }
+__device__ inline float offset_value(double v) { return (float)v; }
+template <typename S>
+__device__ inline void choose_plan(const PlanChoice& pc, const S* __restrict__ off, size_t n) {
+    __shared__ unsigned s_cnt[MAX_PLANS + 1];
+    if (threadIdx.x <= MAX_PLANS) s_cnt[threadIdx.x] = 0;
+    __syncthreads();
+    constexpr unsigned RUN = 256, RUNS = 32;
+    // counted per wavefront (ballots), so that only one lane of each adds to the shared counters
+    unsigned cnt[MAX_PLANS] = {}, seen = 0;
+    auto look = [&](float f, bool there) {
+        seen += (unsigned)__popcll(__ballot(there));
+#pragma unroll
+        for (int k = 0; k < MAX_PLANS; ++k)
+            cnt[k] += (unsigned)__popcll(__ballot(there && !(f >= -(float)pc.margin[k] && f < (float)pc.margin[k])));
+    };
+    if (n <= (size_t)RUN * RUNS) {
+        for (size_t i0 = 0; i0 < n; i0 += blockDim.x) {
+            const size_t i = i0 + threadIdx.x;
+            const bool there = i < n;
+            look(there ? offset_value(off[i]) : 0.f, there);
+        }
+    } else {
+        // all loads of a thread in flight at once: one memory latency, not one per run
+        const size_t step = (n - RUN) / (RUNS - 1);
+        const bool there = threadIdx.x < RUN;
+        const unsigned t = there ? threadIdx.x : 0u;
+        S v[RUNS];
+#pragma unroll
+        for (unsigned r = 0; r < RUNS; ++r) v[r] = off[(size_t)r * step + t];
+#pragma unroll
+        for (unsigned r = 0; r < RUNS; ++r) look(offset_value(v[r]), there);
+    }
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+        for (int k = 0; k < MAX_PLANS; ++k) atomicAdd(&s_cnt[k], cnt[k]);
+        atomicAdd(&s_cnt[MAX_PLANS], seen);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float total = (float)max(s_cnt[MAX_PLANS], 1u);
+        unsigned best = 0;
+        float best_cost = 0.f;
+        for (int k = 0; k < pc.nplans && k < MAX_PLANS; ++k) {
+            const float keep = 1.f - (float)s_cnt[k] / total;             // entries inside the margin
+            float in_sample = keep;
+            for (int a = 1; a < pc.nd; ++a) in_sample *= keep;
+            float in_wave = in_sample;
+            for (int d = 0; d < 6; ++d) in_wave *= in_wave;               // ^64
+            const float cost = pc.base[k] * (1.f + pc.far_wave * (1.f - in_wave) + pc.far_sample * (1.f - in_sample));
+            if (k == 0 || cost < best_cost) { best = (unsigned)k; best_cost = cost; }
+        }
+        *pc.sel = best;
+    }
+}
+
 // WIDE (float, CCH = 8): row j of a pass holds (tap, channel) = (2 * (j / 16) + (j / 4) % 2,
 // 4 * ((j / 8) % 2) + j % 4) instead of (j / CCH, j % CCH): the MFMA then leaves all eight channels
 // of a tap in one lane (fused_row_tap / fused_row_channel).
 // `bounds` (two floats, may be null) is cleared for the weight_bounds_kernel that follows.
+// With pc.sel set the launch has one block more, which chooses the halo plan from the offsets.
 template <typename T, int CCH, bool WIDE = false>
-__global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp, float* __restrict__ bounds) {
+__global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp, float* __restrict__ bounds,
+                                   PlanChoice pc, const T* __restrict__ off, size_t n_off) {
     using MM = Mma<T>;
+    const unsigned pack_blocks = pc.sel ? gridDim.x - 1 : gridDim.x;
+    if (blockIdx.x == pack_blocks) {
+        choose_plan(pc, off, n_off);
+        return;
+    }
     if (bounds && blockIdx.x == 0 && threadIdx.x < 2) bounds[threadIdx.x] = 0.f;
     constexpr int TN = MM::TN, KL = MM::KL, TP = TN / CCH;
     const int npass = (P.kV + TP - 1) / TP;
     const int kst = ((P.M + KL - 1) / KL + 15) / 16 * 16;       // operand batches are 8 or 16 reduction steps
     const size_t per_chunk = (size_t)npass * kst * 64;
     const size_t total = (size_t)chunk_candidates<CCH>(P.cpg, P.Cg, P.C_in) * per_chunk;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)pack_blocks * blockDim.x) {
         const int c0 = chunk_candidate<CCH>(P.cpg, P.Cg, (int)(i / per_chunk));      // candidate first channel of a chunk
         const int seg_b = max(c0 / P.cpg * P.cpg, c0 / P.Cg * P.Cg);
         if ((c0 - seg_b) % CCH) continue;
@@ -199,7 +268,7 @@ struct TileGeo {
 };
 
 template <int ND>
-__device__ inline void tile_decode(const Params& P, unsigned bid, TileGeo<ND>& tg) {
+__device__ inline void tile_decode(const Params& P, const HaloPlan& H, unsigned bid, TileGeo<ND>& tg) {
     unsigned t = bid % (unsigned)P.tiles;
     tg.n = bid / (unsigned)P.tiles;
 #pragma unroll
@@ -208,7 +277,7 @@ __device__ inline void tile_decode(const Params& P, unsigned bid, TileGeo<ND>& t
         const int ti = t % P.ntile[s];
         t /= P.ntile[s];
         tg.o0[a] = ti * P.tdim[s];
-        tg.hb[a] = tg.o0[a] * P.stride[s] - P.pad[s] - P.mlo[s];
+        tg.hb[a] = tg.o0[a] * P.stride[s] - P.pad[s] - H.mlo[s];
     }
 }
 
@@ -237,8 +306,8 @@ __device__ inline bool tile_position(const Params& P, const TileGeo<ND>& tg, int
 // where the halo sticks out of the volume.  Built once per workgroup into LDS (hvol entries) so
 // that staging, zeroing and flushing need no per-thread index math and no registers.
 template <int ND, int WGS = WGH>
-__device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsigned* __restrict__ sTab) {
-    for (int v0 = threadIdx.x; v0 < P.hvol; v0 += WGS) {
+__device__ inline void halo_table(const Params& P, const HaloPlan& H, const TileGeo<ND>& tg, unsigned* __restrict__ sTab) {
+    for (int v0 = threadIdx.x; v0 < H.hvol; v0 += WGS) {
         int v = v0;
         bool inb = true;
         unsigned lin = 0;
@@ -246,8 +315,8 @@ __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsign
 #pragma unroll
         for (int a = ND - 1; a >= 0; --a) {
             const int s = slot<ND>(a);
-            c[a] = tg.hb[a] + v % P.hext[s];
-            v /= P.hext[s];
+            c[a] = tg.hb[a] + v % H.hext[s];
+            v /= H.hext[s];
             inb = inb && c[a] >= 0 && c[a] < P.in[s];
         }
 #pragma unroll
@@ -260,9 +329,9 @@ __device__ inline void halo_table(const Params& P, const TileGeo<ND>& tg, unsign
 // next to each other, so one wide LDS read fetches a corner of all of them (missing channels of a
 // short last chunk and halo voxels outside the volume are stored as zero).
 template <typename T, int CCH, int WGS>
-__device__ inline void halo_stage_interleaved(const Params& P, const T* __restrict__ chan0, int nch,
+__device__ inline void halo_stage_interleaved(const Params& P, const HaloPlan& H, const T* __restrict__ chan0, int nch,
                                               const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
-    for (int v = threadIdx.x; v < P.hvol; v += WGS) {
+    for (int v = threadIdx.x; v < H.hvol; v += WGS) {
         const unsigned t = sTab[v];
         const unsigned g = t == ~0u ? 0u : t;
         T val[CCH];
@@ -336,6 +405,8 @@ struct Fp16 {       // IEEE binary16
     __device__ static inline float widen(Fp16 x) { return (float)x.v; }
     __device__ static inline Fp16 narrow(float f) { Fp16 r; r.v = (_Float16)f; return r; }
 };
+__device__ inline float offset_value(Bf16 v) { return Bf16::widen(v); }
+__device__ inline float offset_value(Fp16 v) { return Fp16::widen(v); }
 template <typename S>
 __global__ void widen_kernel(const S* __restrict__ src, float* __restrict__ dst, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::widen(src[i]);
@@ -733,13 +804,16 @@ __global__ __launch_bounds__(512) void weight_bounds_kernel(const T* __restrict_
 // -- still fit 31 bits; the host allows it only while that leaves enough bits below that term.
 // wmax[1] then holds the largest column norm of the weight (colnorm_max_kernel).
 template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false, int BS = 1>
-__global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, const T* __restrict__ in,
+__global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
+                                                                  const T* __restrict__ in,
                                                                   const T* __restrict__ off,
                                                                   const T* __restrict__ Wt,
                                                                   const T* __restrict__ gout,
                                                                   const float* __restrict__ wmax,
                                                                   T* __restrict__ gin, T* __restrict__ goff, int csplit,
                                                                   unsigned whole, int goff_atomic) {
+    HaloPlan H;
+    if (!chosen_halo(P, alts, sel, H)) return;          // another launch runs the chosen plan
     using MM = Mma<T>;
     using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
@@ -758,7 +832,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     static_assert(!PAIR || (sizeof(T) == 4 && RPS % 2 == 0), "paired cells are a float32 layout");
     constexpr int CPL = PAIR ? CCH / 2 : CCH;           // cell planes
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const int hs = HS ? HS : P.hstride;
+    const int hs = HS ? HS : H.hstride;
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CPL][hstride]
     T* sIn = reinterpret_cast<T*>(sG + (size_t)CPL * hs);                               // [hstride][CCH] if COORD: channels of a voxel side by side
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
@@ -785,14 +859,14 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     const int dg = item / nt;
 
     TileGeo<ND> tg;
-    tile_decode<ND>(P, item % nt, tg);
+    tile_decode<ND>(P, H, item % nt, tg);
     const int n = tg.n;
     int o[ND], ib[ND];
     unsigned pos;
     const bool valid = tile_position<ND>(P, tg, wave * TN + j, o, pos);
 #pragma unroll
     for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
-    halo_table<ND, WGS>(P, tg, sTab);                   // visible after the first barrier below
+    halo_table<ND, WGS>(P, H, tg, sTab);                  // visible after the first barrier below
     // o * stride - pad of this lane's position as T: the integer part of a sampling coordinate is
     // (T)(that + tap * dilation), a sum of two small integers that is exact in T as well
     T ibf[ND];
@@ -906,8 +980,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             const int nch = min(CCH, re - cc0);
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < (PAIR ? (nch + 1) / 2 : nch); ++c)
-                for (int v = threadIdx.x; v < P.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
-            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
+                for (int v = threadIdx.x; v < H.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
+            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, H, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
             __syncthreads();
 
             // Grad-column tile of a pass: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past
@@ -1071,8 +1145,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             unsigned coff[NC];
 #pragma unroll
             for (int i = 0; i < NC; ++i)
-                coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * P.hext[1] + ((i >> 1) & 1)) * P.hext[2] + (i & 1))
-                                  : (unsigned)(((i >> 1) & 1) * P.hext[2] + (i & 1));
+                coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * H.hext[1] + ((i >> 1) & 1)) * H.hext[2] + (i & 1))
+                                  : (unsigned)(((i >> 1) & 1) * H.hext[2] + (i & 1));
 
             for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
                 const typename MM::Acc d = d_next;
@@ -1127,12 +1201,12 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         inside = inside && fabs(pa - pc) < (T)1;            // -1 < p < size, false for NaN
                         intr[a] = pa > (T)0 && pa < top;
                         u[a] = (int)fl - tg.hb[a];
-                        inhalo = inhalo && (unsigned)u[a] < (unsigned)(P.hext[s] - 1);
+                        inhalo = inhalo && (unsigned)u[a] < (unsigned)(H.hext[s] - 1);
                     }
                     const bool near = inside && inhalo, far = inside && !inhalo;
                     unsigned base;
-                    if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], P.hext[1]) + u[1], P.hext[2]) + u[2]);
-                    else base = (unsigned)(__mul24(u[0], P.hext[2]) + u[1]);
+                    if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], H.hext[1]) + u[1], H.hext[2]) + u[2]);
+                    else base = (unsigned)(__mul24(u[0], H.hext[2]) + u[1]);
                     base = near ? base : 0u;       // lanes without a sample in the halo read cell 0 and add nothing
                     T cw[NC];
                     if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
@@ -1322,7 +1396,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             if constexpr (COORD) write_goff();
             first_chunk = false;
             __syncthreads();                        // all LDS adds of this chunk have landed
-            for (int v = threadIdx.x; v < P.hvol; v += WGS) {
+            for (int v = threadIdx.x; v < H.hvol; v += WGS) {
                 const unsigned gv = sTab[v];
                 if (gv == ~0u) continue;            // halo cell outside the volume: never touched
                 if constexpr (PAIR) {
