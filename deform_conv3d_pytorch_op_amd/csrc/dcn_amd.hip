@@ -535,7 +535,10 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
             pc.nd = ND;
             pc.margin[0] = margins[0];
             pc.base[0] = 1.f;
-            pc.far_wave = 1.5f;             // a wavefront with a sample beyond the halo gathers every channel of the pass from global memory
+            // a wavefront with a sample beyond the halo walks every channel of the pass once more, and each
+            // such sample gathers its corners from global memory (fitted to timings at c4 and c3)
+            pc.far_wave = ND == 3 ? 0.5f : 0.1f;
+            pc.far_sample = ND == 3 ? 2.2f : 5.f;
             const size_t used = align256(wq_bytes) + (fsplit > 1 ? (size_t)fsplit * out_bytes : 0);
             if (nmargins > 1 && ws_bytes >= used + 512) {
                 // (within the LDS of the first plan, which fixes how many workgroups share a CU; all of it
@@ -550,8 +553,8 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                     if (!same_blocks(Pk, plans[0]) || Pk.hvol > 3 * plans[0].hvol) continue;
                     if (fsplit > 1) even_passes(Pk);
                     pc.margin[pc.nplans] = margins[k];
-                    // staging and the per-pass geometry grow with the halo: about half of the kernel's time in 3-D, an eighth in 2-D
-                    pc.base[pc.nplans] = 1.f + (ND == 3 ? 0.5f : 0.12f) * ((float)Pk.hvol / (float)plans[0].hvol - 1.f);
+                    // staging and the per-pass geometry grow with the halo: about a third of the kernel's time in 3-D, an eighth in 2-D
+                    pc.base[pc.nplans] = 1.f + (ND == 3 ? 0.3f : 0.12f) * ((float)Pk.hvol / (float)plans[0].hvol - 1.f);
                     ++pc.nplans;
                 }
                 if (pc.nplans > 1) pc.sel = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + (ws_bytes - 256) / 256 * 256);
@@ -800,7 +803,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         fp[0].wt = wt;
         for (int k = 1; k < nmargins; ++k) {
             FusedPlan& c = fp[pc.nplans];
-            if (!plan_fused(margins[k], c) || c.nw != fp[0].nw || c.Ph.hvol > 3 * fp[0].Ph.hvol) continue;
+            if (!plan_fused(margins[k], c) || c.Ph.hvol > 3 * fp[0].Ph.hvol) continue;
             for (int e = 0; e < pc.nplans && !c.wt; ++e)
                 if (fp[e].cch == c.cch && fp[e].wide == c.wide) c.wt = fp[e].wt;
             if (!c.wt) {
@@ -810,7 +813,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             }
             pc.margin[pc.nplans] = margins[k];
             // flush, staging and the per-chunk passes grow with the halo: most of the kernel's time in 3-D, little in 2-D
-            pc.base[pc.nplans] = 1.f + (ND == 3 ? 0.9f : 0.05f) * ((float)c.Ph.hvol / (float)fp[0].Ph.hvol - 1.f);
+            // (a quarter more where only the shape with half the wavefronts fits)
+            pc.base[pc.nplans] = (1.f + (ND == 3 ? 0.9f : 0.05f) * ((float)c.Ph.hvol / (float)fp[0].Ph.hvol - 1.f)) * (c.nw < fp[0].nw ? 1.25f : 1.f);
             ++pc.nplans;
         }
         for (int k = pc.nplans; k < MAX_PLANS; ++k) {
