@@ -65,7 +65,9 @@ const char *dcn_last_error(void);   /* message of the last failing call on this 
  * 16-bit formats, elem_size 2, are served by dcn_workspace_bytes_for only and get 0 here;
  * input_volume = input_l * input_h * input_w, output_volume likewise, kernel_volume =
  * kernel_l * kernel_h * kernel_w).  The workspace holds a re-laid-out copy of the weight and, for
- * the backward calls, channels-last copies of the input batch, its gradient and grad_output. */
+ * the backward calls, channels-last copies of the input batch, its gradient and grad_output, and
+ * one word in which the device records which of the planned LDS halo sizes it chose for the call
+ * from the offsets (so two calls that overlap in time need a workspace each). */
 size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
                            size_t output_volume, int kernel_volume, int group);
 /* The same for a known number of channels per deformable group (the reference's
@@ -103,7 +105,8 @@ int dcn3d_backward_input_offset_f64(const double *input, const double *weight, c
  * is for callers that cannot allocate device memory around the call (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  Same arguments, results and kernels as
  * dcn3d_forward_f32 without the workspace pair; the re-laid-out weight (and, for a layer of few
- * positions, as many partial outputs as still fit) goes into a fixed device array
+ * positions, as many partial outputs as still fit; in the last 256 bytes the halo size chosen for
+ * the call) goes into a fixed device array
  * of DCN_NOALLOC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until
  * the process ends.  A layer whose re-laid-out weight is larger (roughly: 4 * kernel volume *
  * output_c rounded up to 256 * (input_c / group + 4) bytes) is rejected with DCN_E_WORKSPACE.  All
