@@ -438,6 +438,41 @@ def test_forward_and_grad_weight_are_deterministic():
         assert rel_err(again[1], first[1].cpu()) < 1e-5 and rel_err(again[2], first[2].cpu()) < 1e-5
 
 
+@pytest.mark.parametrize("nd", [2, 3])
+def test_halo_plan_follows_the_offsets(nd):
+    """The forward call records which of its planned LDS halo sizes the device chose, as a 32-bit
+    index in the workspace at byte offset (workspace_bytes - 256) rounded down to a multiple of 256
+    (include/dcn_amd.h): plan 0, margin 2, for offsets within +-1; plan 1 (margin 3, in 2-D 4) for
+    offsets up to +-2.6, of which a fifth reach past +-2; plan 2 (margin 4, in 2-D 6) for offsets
+    up to +-3.7 (+-5.9).  The output agrees with the oracle whichever plan runs."""
+    if os.environ.get("DCN_HALO_MARGIN") or os.environ.get("DCN_ADAPTIVE_MARGIN") == "0":
+        pytest.skip("one fixed halo margin is forced: nothing is chosen")
+    from deform_conv3d_pytorch_op_amd import _lib
+    from deform_conv3d_pytorch_op_amd.functions import _geom
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    spec = (3, 2, 16, 16, (8, 16, 24), 3, 1, 1, 1, 8, 1) if nd == 3 else (2, 2, 32, 16, (40, 48), 3, 1, 1, 1, 16, 1)
+    chosen = {}
+    for label, scale in (("narrow", 1.0), ("wide", 2.6), ("widest", 3.7 if nd == 3 else 5.9)):
+        print("halo plan", nd, label, flush=True)
+        c = make_case(*spec, scale, dtype=torch.float32, seed=21, bias=False)
+        x, off, w = (c[k].to(dev) for k in ("x", "off", "w"))
+        geom = _geom(nd, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+        nbytes = L.dcn_workspace_bytes_for(4, x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]), math.prod(c["outs"]),
+                                           math.prod(c["k"]), c["groups"], c["cpg"])
+        ws = torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=dev)
+        out = torch.empty((x.shape[0], w.shape[0]) + c["outs"], dtype=torch.float32, device=dev)
+        rc = getattr(L, "dcn%dd_forward_f32" % nd)(x.data_ptr(), w.data_ptr(), off.data_ptr(), None, out.data_ptr(), *geom,
+                                                   ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, L.dcn_last_error()
+        torch.cuda.synchronize()
+        at = (nbytes - 256) // 256 * 256
+        chosen[label] = int.from_bytes(bytes(ws[at:at + 4].cpu().tolist()), "little")
+        want = orc.forward(c["x"], c["off"], c["w"], None, c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+        assert rel_err(out, want) < TOL[torch.float32]["fwd"], label
+    assert chosen == {"narrow": 0, "wide": 1, "widest": 2}, chosen
+
+
 def test_hip_graph_replay():
     """Forward + backward captured into a HIP graph (the C ABI allocates nothing, clears memory with
     kernels only and never synchronises); every replay, with eager work and synchronisations in
