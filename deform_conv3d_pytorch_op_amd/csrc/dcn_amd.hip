@@ -182,6 +182,8 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_LDS_BUDGET_KB      LDS per 512-thread workgroup of the forward halo kernel (default 72: two per CU)
 //   DCN_FORWARD_WG=512     never use the 1024-thread forward variant; =1024 use it whenever its halo fits
 //   DCN_FORWARD_SPLIT=n    forward pass: split the input channels of a position block over at most n workgroups (0: never)
+//   DCN_FORWARD_TAIL=0     forward pass: never split only the units of the last, partly filled round of workgroups (n > 1: n ways)
+//   DCN_FORWARD_SLOTS=n    forward pass: plan the launch as if n workgroups ran at once (test hook)
 //   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
@@ -265,6 +267,14 @@ static int forced_slots() {             // DCN_FUSED_SLOTS=n (test hook): plan t
 }
 static int forward_split() {            // DCN_FORWARD_SPLIT=n: the forward pass splits the input channels of a position block at most n ways
     static const int v = [] { const char* e = getenv("DCN_FORWARD_SPLIT"); return e ? atoi(e) : 1 << 20; }();
+    return v;
+}
+static int forward_slots() {            // DCN_FORWARD_SLOTS=n (test hook): plan the forward launch as if n workgroups ran at once
+    static const int v = [] { const char* e = getenv("DCN_FORWARD_SLOTS"); return e && atoi(e) > 0 ? atoi(e) : 0; }();
+    return v;
+}
+static int forward_tail_split() {       // DCN_FORWARD_TAIL=0: the forward pass never splits the units of its last round of workgroups; n > 1: n ways
+    static const int v = [] { const char* e = getenv("DCN_FORWARD_TAIL"); return e ? atoi(e) : 1; }();
     return v;
 }
 static bool fused_pair() {              // DCN_FUSED_PAIR=0: float32 LDS cells of the fused backward kernel hold one channel each (64-bit)
@@ -580,31 +590,65 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                 if (l > lds) lds = l;
             }
             const Params& Ph = plans[0];
-            const dim3 grid((unsigned)Ph.N * Ph.tiles * Ph.G * Ph.mchunks * fsplit);
+            using Kern = void (*)(Params, PlanSet, const unsigned*, const S*, const S*, const S*, const S*, S*, S*, int, unsigned);
+            Kern kern;
+            if (nw == 16) kern = MT == 1 ? forward_quad_kernel<T, ND, 1, 16, S> : forward_quad_kernel<T, ND, 2, 16, S>;
+            else kern = MT == 1 ? forward_quad_kernel<T, ND, 1, WAVESH, S> : MT == 2 ? forward_quad_kernel<T, ND, 2, WAVESH, S>
+                      : MT == 4 ? forward_quad_kernel<T, ND, 4, WAVESH, S> : forward_quad_kernel<T, ND, 8, WAVESH, S>;
+            S* part = reinterpret_cast<S*>(static_cast<char*>(ws) + align256(wq_bytes));
+            // A grid that ends in a partly filled round of workgroups: the units of that round, last in
+            // the launch, are split over tsplit workgroups each (every tsplit-th channel pass), so that
+            // the round fills the device; forward_join_tail_kernel adds their partial sums.  A
+            // workgroup's fixed part (halo table, offsets, output) is charged as 5 % of a unit.
+            const long long units = (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks;
+            int tsplit = 1;
+            long long whole = 0;
+            if (!S16 && fsplit == 1 && forward_tail_split()) {
+                const long long slots = forward_slots() ? forward_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
+                const long long rest = units % slots;
+                int passes = 0;                 // channel passes of a unit under the first plan
+                for (int dg = 0; dg <= (P.Cg - 1) / P.cpg; ++dg) {
+                    const int len = (P.Cg < (dg + 1) * P.cpg ? P.Cg : (dg + 1) * P.cpg) - dg * P.cpg;
+                    passes += (len + Ph.cchunk - 1) / Ph.cchunk;
+                }
+                const size_t end = pc.sel ? (ws_bytes - 256) / 256 * 256 : ws_bytes;
+                const size_t room = end > align256(wq_bytes) ? end - align256(wq_bytes) : 0;
+                if (units > slots && rest) {
+                    double best = 0.9;          // of the time of an unsplit last round; a tenth must be gained
+                    for (int cs = 2; cs <= 8 && cs <= passes; ++cs) {
+                        const double t = (double)((rest * cs + slots - 1) / slots) * ((double)((passes + cs - 1) / cs) / passes + 0.05);
+                        const size_t bytes = (size_t)rest * cs * MT * TN * nw * TN * sizeof(T);
+                        if (forward_tail_split() > 1 && cs != forward_tail_split()) continue;
+                        if ((t < best || forward_tail_split() > 1) && bytes <= room && bytes <= FWD_PARTIAL_CAP) { best = t; tsplit = cs; }
+                    }
+                    if (tsplit > 1) whole = units - rest;
+                }
+            }
+            const long long wgs = tsplit > 1 ? whole + (units - whole) * tsplit : units * fsplit;
+            if (wgs > 0x7fffffffLL) return fail(DCN_E_ARGUMENT, "too many workgroups for one launch");
+            const dim3 grid((unsigned)wgs);
             if (trace_plans()) {
-                fprintf(stderr, "dcn forward: %d wavefronts, MT %d, grid %u, LDS %zu, split %d\n", nw, MT, grid.x, lds, fsplit);
+                fprintf(stderr, "dcn forward: %d wavefronts, MT %d, grid %u (%lld unsplit, rest x %d), LDS %zu, every unit split x %d\n", nw, MT, grid.x,
+                        tsplit > 1 ? whole : 0LL, tsplit, lds, fsplit);
                 for (int k = 0; k < pc.nplans; ++k)
                     fprintf(stderr, "  plan %d: margin %d, halo %d x %d x %d, %d channels per pass, base cost %.3f\n", k, pc.margin[k],
                             plans[k].hext[0], plans[k].hext[1], plans[k].hext[2], plans[k].cchunk, pc.base[k]);
             }
-            S* part = reinterpret_cast<S*>(static_cast<char*>(ws) + align256(wq_bytes));
-            S* dst = fsplit > 1 ? part : out;
-            const S* kbias = fsplit > 1 ? nullptr : bias;
             const unsigned* sel = pc.sel;
-            int rc;
-            if (nw == 16) {
-                rc = MT == 1 ? launch_halo(forward_quad_kernel<T, ND, 1, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit)
-                             : launch_halo(forward_quad_kernel<T, ND, 2, 16, S>, "forward_quad_kernel", grid, 1024, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit);
-            } else {
-                switch (MT) {
-                    case 1: rc = launch_halo(forward_quad_kernel<T, ND, 1, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
-                    case 2: rc = launch_halo(forward_quad_kernel<T, ND, 2, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
-                    case 4: rc = launch_halo(forward_quad_kernel<T, ND, 4, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
-                    default: rc = launch_halo(forward_quad_kernel<T, ND, 8, WAVESH, S>, "forward_quad_kernel", grid, WGH, lds, s, Ph, alts, sel, in, off, wt, kbias, dst, fsplit); break;
-                }
-            }
-            if (rc || fsplit == 1) return rc;
+            if (int rc = launch_halo(kern, "forward_quad_kernel", grid, nw * 64, lds, s, Ph, alts, sel, in, off, (const S*)wt, bias, out, part,
+                                     tsplit > 1 ? tsplit : fsplit, (unsigned)whole))
+                return rc;
+            if (fsplit == 1 && tsplit == 1) return DCN_OK;
             if constexpr (!S16) {
+                if (tsplit > 1) {
+                    using Join = void (*)(Params, PlanSet, const unsigned*, const T*, const T*, T*, int, unsigned);
+                    Join join;
+                    if (nw == 16) join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, 16> : forward_join_tail_kernel<T, ND, 2, 16>;
+                    else join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, WAVESH> : MT == 2 ? forward_join_tail_kernel<T, ND, 2, WAVESH>
+                              : MT == 4 ? forward_join_tail_kernel<T, ND, 4, WAVESH> : forward_join_tail_kernel<T, ND, 8, WAVESH>;
+                    hipLaunchKernelGGL(join, dim3((unsigned)(units - whole)), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole);
+                    return check_launch("forward_join_tail_kernel");
+                }
                 const size_t total = (size_t)P.N * P.C_out * P.outV;
                 const unsigned jb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
                 hipLaunchKernelGGL(forward_join_partials_kernel<T>, dim3(jb), dim3(256), 0, s, part, bias, out, fsplit, total, P.C_out, P.outV);

@@ -117,10 +117,16 @@ __device__ inline void halo_stage_quads(const Params& P, const HaloPlan& H, cons
 
 // 1-D grid of N * tiles (blocks of positions) * G * mchunks * csplit workgroups of NW wavefronts;
 // dynamic LDS = cchunk * hstride * sizeof(T) + hvol * 4 with cchunk a multiple of four.
-// csplit > 1 (layers with too few position blocks to fill the device): the csplit workgroups of a
-// (block, group, output-channel chunk) share its input-channel chunks -- workgroup cz takes every
-// csplit-th -- and write their partial sums, without bias, to out + cz * N * C_out * outV;
-// forward_join_partials_kernel adds them up in a fixed order.
+// csplit > 1: csplit workgroups share the input-channel chunks of a unit (block, group,
+// output-channel chunk) -- workgroup cz takes every csplit-th -- and write partial sums without
+// bias, which a second kernel adds up in a fixed order.  Two uses:
+//   whole = 0 (layers with too few position blocks to fill the device): every unit is split; the
+//     partial outputs are whole output tensors at part + cz * N * C_out * outV
+//     (forward_join_partials_kernel);
+//   whole > 0 (a grid that ends in a partly filled round of workgroups): the first `whole` units
+//     run unsplit and write the output itself, the others, last in the launch, are split so that
+//     the last round fills the device; their partial sums go to part as
+//     [unit - whole][cz][row of the chunk][position of the block] (forward_join_tail_kernel).
 // (few accumulators: four wavefronts per SIMD, i.e. at most 128 registers, also for the 512-thread
 // shape, so that two of its workgroups share a CU)
 // S: storage format of the tensors (see Store); with a 16-bit format T is float and csplit must be 1.
@@ -128,7 +134,8 @@ template <typename T, int ND, int MT, int NW, typename S = T>
 __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
                                                            const S* __restrict__ in,
                                                            const S* __restrict__ off, const S* __restrict__ Wq,
-                                                           const S* __restrict__ bias, S* __restrict__ out, int csplit) {
+                                                           const S* __restrict__ bias, S* __restrict__ out,
+                                                           S* __restrict__ part, int csplit, unsigned whole) {
     HaloPlan H;
     if (!chosen_halo(P, alts, sel, H)) return;          // another launch runs the chosen plan
     using MM = Mma<T>;
@@ -141,9 +148,16 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     // workgroups of one tile are neighbours in an XCD-contiguous order
-    const unsigned wgs = xcd_contiguous(blockIdx.x, gridDim.x);
-    const int cz = wgs % (unsigned)csplit;
-    const unsigned wg = wgs / (unsigned)csplit;
+    unsigned wg;
+    int cz = 0;
+    const bool split = csplit > 1 && blockIdx.x >= whole;
+    if (!split) wg = xcd_contiguous(blockIdx.x, csplit > 1 ? whole : gridDim.x);
+    else {
+        const unsigned r = xcd_contiguous(blockIdx.x - whole, gridDim.x - whole);
+        wg = whole + r / (unsigned)csplit;
+        cz = r % (unsigned)csplit;
+    }
+    if (!split) csplit = 1;
     const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
     const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
 
@@ -360,8 +374,18 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
         }
     }
 
+    if (split && whole > 0) {
+        // partial sums of a unit of the last round: [unit - whole][cz][MT * TN rows][NW * TN positions]
+        S* dst = part + ((size_t)(wg - whole) * csplit + cz) * (MT * TN) * (NW * TN) + wave * TN + j;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < MM::NACC; ++r) dst[(size_t)(mt * TN + MM::row(r, q)) * (NW * TN)] = Store<S>::st(acc[mt][r]);
+        return;
+    }
     if (!valid) return;
-    S* dst = out + (size_t)cz * P.N * P.C_out * P.outV;
+    // unsplit: the output with bias; every unit split: a partial output tensor per cz, the bias is added when they are joined
+    S* dst = split ? part + (size_t)cz * P.N * P.C_out * P.outV : out;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -369,10 +393,40 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
             const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
             if (m < P.M) {
                 T v = acc[mt][r];
-                if (bias) v += Store<S>::ld(bias[g * P.M + m]);
+                if (bias && !split) v += Store<S>::ld(bias[g * P.M + m]);
                 dst[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = Store<S>::st(v);
             }
         }
+}
+
+// Joins the partial sums of the units that forward_quad_kernel split in its last round: one
+// workgroup of NW * TN threads per unit, thread = position of the block; out = bias + the csplit
+// partial sums, added in the order of cz.
+template <typename T, int ND, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
+                                                                    const T* __restrict__ part, const T* __restrict__ bias,
+                                                                    T* __restrict__ out, int csplit, unsigned whole) {
+    constexpr int TN = Mma<T>::TN;
+    HaloPlan H;
+    if (!chosen_halo(P, alts, sel, H)) return;
+    if (threadIdx.x >= NW * TN) return;
+    const unsigned wg = whole + blockIdx.x;
+    const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
+    const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
+    TileGeo<ND> tg_;
+    tile_decode<ND>(P, H, wg / (unsigned)(P.G * P.mchunks), tg_);
+    int o[ND];
+    unsigned pos;
+    if (!tile_position<ND>(P, tg_, (int)threadIdx.x, o, pos)) return;
+    const T* src = part + (size_t)blockIdx.x * csplit * (MT * TN) * (NW * TN) + threadIdx.x;
+    for (int ml = 0; ml < MT * TN; ++ml) {
+        const int m = mchunk * MT * TN + ml;
+        if (m >= P.M) break;
+        T v = src[(size_t)ml * (NW * TN)];
+        for (int cz = 1; cz < csplit; ++cz) v += src[((size_t)cz * (MT * TN) + ml) * (NW * TN)];
+        if (bias) v += bias[g * P.M + m];
+        out[((size_t)tg_.n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+    }
 }
 
 // out = bias + the sum of `parts` partial outputs of forward_quad_kernel, added in the order of the

@@ -17,6 +17,9 @@ settings, each in a process of its own (the knobs are read once per process):
   DCN_OVERLAP_BACKWARD=1  backward_weight on a second stream next to backward_input_offset
   DCN_FUSED_BREG2=0    the grad_output operand of 64 < M <= 128 output channels read from memory instead of a second register set
   DCN_FUSED_PAIR=0     float32 LDS cells of the fused backward kernel with one channel each (64-bit) instead of two
+  DCN_FORWARD_SLOTS=3  plans the forward launch for a device of three workgroups: the units of the last, partly filled
+                       round are split over workgroups whose partial sums a second kernel joins (otherwise only
+                       full-size layers get there); DCN_FORWARD_TAIL=2 forces a two-way split, =0 none
   DCN_ADAPTIVE_MARGIN=0  one halo margin of 2 instead of the choice on the device among 2, 3, 4 (2, 4, 6 in 2-D): the
                        cases with wide offsets then take the paths through global memory (the default runs cover the
                        wider plans and the choice)
@@ -46,6 +49,10 @@ SETTINGS = [
     {"DCN_FUSED_SLOTS": "3", "DCN_FUSED_TAIL": "0", "DCN_FUSED_FIXED": "0"},
     {"DCN_OVERLAP_BACKWARD": "1", "DCN_FORWARD_SPLIT": "0"},
     {"DCN_FUSED_PAIR": "0", "DCN_FUSED_BREG2": "0"},
+    # the forward pass planned for a device of three workgroups: units of the last round split over several workgroups
+    {"DCN_FORWARD_SLOTS": "3"},
+    {"DCN_FORWARD_SLOTS": "5", "DCN_FORWARD_TAIL": "2", "DCN_FORWARD_SPLIT": "0"},
+    {"DCN_FORWARD_TAIL": "0"},
     # one halo margin, as narrow as the default: the wide offsets of the cases then leave the halo
     # and take the paths through global memory, which the margin chosen on the device avoids
     {"DCN_ADAPTIVE_MARGIN": "0"},
