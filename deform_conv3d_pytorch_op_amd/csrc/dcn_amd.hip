@@ -646,7 +646,7 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                     if (nw == 16) join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, 16> : forward_join_tail_kernel<T, ND, 2, 16>;
                     else join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, WAVESH> : MT == 2 ? forward_join_tail_kernel<T, ND, 2, WAVESH>
                               : MT == 4 ? forward_join_tail_kernel<T, ND, 4, WAVESH> : forward_join_tail_kernel<T, ND, 8, WAVESH>;
-                    hipLaunchKernelGGL(join, dim3((unsigned)(units - whole)), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole);
+                    hipLaunchKernelGGL(join, dim3((unsigned)((units - whole) * (MT * TN / JOIN_ROWS))), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole);
                     return check_launch("forward_join_tail_kernel");
                 }
                 const size_t total = (size_t)P.N * P.C_out * P.outV;

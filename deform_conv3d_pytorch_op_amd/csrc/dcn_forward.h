@@ -400,17 +400,20 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
 }
 
 // Joins the partial sums of the units that forward_quad_kernel split in its last round: one
-// workgroup of NW * TN threads per unit, thread = position of the block; out = bias + the csplit
-// partial sums, added in the order of cz.
+// workgroup of NW * TN threads per unit and slice of JOIN_ROWS output channels, thread = position of
+// the block; out = bias + the csplit partial sums, added in the order of cz.
+constexpr int JOIN_ROWS = 8;
 template <typename T, int ND, int MT, int NW>
 __global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
                                                                     const T* __restrict__ part, const T* __restrict__ bias,
                                                                     T* __restrict__ out, int csplit, unsigned whole) {
-    constexpr int TN = Mma<T>::TN;
+    constexpr int TN = Mma<T>::TN, SLICES = MT * TN / JOIN_ROWS;
+    static_assert(MT * TN % JOIN_ROWS == 0, "row slices");
     HaloPlan H;
     if (!chosen_halo(P, alts, sel, H)) return;
     if (threadIdx.x >= NW * TN) return;
-    const unsigned wg = whole + blockIdx.x;
+    const unsigned unit = blockIdx.x / SLICES, ml0 = (blockIdx.x % SLICES) * JOIN_ROWS;
+    const unsigned wg = whole + unit;
     const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
     const int g = gm / P.mchunks, mchunk = gm % P.mchunks;
     TileGeo<ND> tg_;
@@ -418,14 +421,21 @@ __global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, Pl
     int o[ND];
     unsigned pos;
     if (!tile_position<ND>(P, tg_, (int)threadIdx.x, o, pos)) return;
-    const T* src = part + (size_t)blockIdx.x * csplit * (MT * TN) * (NW * TN) + threadIdx.x;
-    for (int ml = 0; ml < MT * TN; ++ml) {
-        const int m = mchunk * MT * TN + ml;
-        if (m >= P.M) break;
-        T v = src[(size_t)ml * (NW * TN)];
-        for (int cz = 1; cz < csplit; ++cz) v += src[((size_t)cz * (MT * TN) + ml) * (NW * TN)];
-        if (bias) v += bias[g * P.M + m];
-        out[((size_t)tg_.n * P.C_out + g * P.M + m) * P.outV + pos] = v;
+    const T* src = part + ((size_t)unit * csplit * (MT * TN) + ml0) * (NW * TN) + threadIdx.x;
+    T v[JOIN_ROWS];
+#pragma unroll
+    for (int r = 0; r < JOIN_ROWS; ++r) v[r] = src[(size_t)r * (NW * TN)];
+    for (int cz = 1; cz < csplit; ++cz) {
+        T a[JOIN_ROWS];
+#pragma unroll
+        for (int r = 0; r < JOIN_ROWS; ++r) a[r] = src[((size_t)cz * (MT * TN) + r) * (NW * TN)];
+#pragma unroll
+        for (int r = 0; r < JOIN_ROWS; ++r) v[r] += a[r];
+    }
+#pragma unroll
+    for (int r = 0; r < JOIN_ROWS; ++r) {
+        const int m = mchunk * MT * TN + (int)ml0 + r;
+        if (m < P.M) out[((size_t)tg_.n * P.C_out + g * P.M + m) * P.outV + pos] = bias ? v[r] + bias[g * P.M + m] : v[r];
     }
 }
 
