@@ -590,12 +590,12 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                 if (l > lds) lds = l;
             }
             const Params& Ph = plans[0];
-            using Kern = void (*)(Params, PlanSet, const unsigned*, const S*, const S*, const S*, const S*, S*, S*, int, unsigned);
+            using Kern = void (*)(Params, PlanSet, const unsigned*, const S*, const S*, const S*, const S*, S*, T*, int, unsigned);
             Kern kern;
             if (nw == 16) kern = MT == 1 ? forward_quad_kernel<T, ND, 1, 16, S> : forward_quad_kernel<T, ND, 2, 16, S>;
             else kern = MT == 1 ? forward_quad_kernel<T, ND, 1, WAVESH, S> : MT == 2 ? forward_quad_kernel<T, ND, 2, WAVESH, S>
                       : MT == 4 ? forward_quad_kernel<T, ND, 4, WAVESH, S> : forward_quad_kernel<T, ND, 8, WAVESH, S>;
-            S* part = reinterpret_cast<S*>(static_cast<char*>(ws) + align256(wq_bytes));
+            T* part = reinterpret_cast<T*>(static_cast<char*>(ws) + align256(wq_bytes));      // partial sums, in the arithmetic type
             // A grid that ends in a partly filled round of workgroups: the units of that round, last in
             // the launch, are split over tsplit workgroups each (every tsplit-th channel pass), so that
             // the round fills the device; forward_join_tail_kernel adds their partial sums.  A
@@ -603,7 +603,7 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
             const long long units = (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks;
             int tsplit = 1;
             long long whole = 0;
-            if (!S16 && fsplit == 1 && forward_tail_split()) {
+            if (fsplit == 1 && forward_tail_split()) {
                 const long long slots = forward_slots() ? forward_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
                 const long long rest = units % slots;
                 int passes = 0;                 // channel passes of a unit under the first plan
@@ -639,16 +639,16 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                                      tsplit > 1 ? tsplit : fsplit, (unsigned)whole))
                 return rc;
             if (fsplit == 1 && tsplit == 1) return DCN_OK;
+            if (tsplit > 1) {
+                using Join = void (*)(Params, PlanSet, const unsigned*, const T*, const S*, S*, int, unsigned);
+                Join join;
+                if (nw == 16) join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, 16, S> : forward_join_tail_kernel<T, ND, 2, 16, S>;
+                else join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, WAVESH, S> : MT == 2 ? forward_join_tail_kernel<T, ND, 2, WAVESH, S>
+                          : MT == 4 ? forward_join_tail_kernel<T, ND, 4, WAVESH, S> : forward_join_tail_kernel<T, ND, 8, WAVESH, S>;
+                hipLaunchKernelGGL(join, dim3((unsigned)((units - whole) * (MT * TN / JOIN_ROWS))), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole);
+                return check_launch("forward_join_tail_kernel");
+            }
             if constexpr (!S16) {
-                if (tsplit > 1) {
-                    using Join = void (*)(Params, PlanSet, const unsigned*, const T*, const T*, T*, int, unsigned);
-                    Join join;
-                    if (nw == 16) join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, 16> : forward_join_tail_kernel<T, ND, 2, 16>;
-                    else join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, WAVESH> : MT == 2 ? forward_join_tail_kernel<T, ND, 2, WAVESH>
-                              : MT == 4 ? forward_join_tail_kernel<T, ND, 4, WAVESH> : forward_join_tail_kernel<T, ND, 8, WAVESH>;
-                    hipLaunchKernelGGL(join, dim3((unsigned)((units - whole) * (MT * TN / JOIN_ROWS))), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole);
-                    return check_launch("forward_join_tail_kernel");
-                }
                 const size_t total = (size_t)P.N * P.C_out * P.outV;
                 const unsigned jb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
                 hipLaunchKernelGGL(forward_join_partials_kernel<T>, dim3(jb), dim3(256), 0, s, part, bias, out, fsplit, total, P.C_out, P.outV);

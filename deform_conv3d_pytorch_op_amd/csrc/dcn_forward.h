@@ -129,13 +129,13 @@ __device__ inline void halo_stage_quads(const Params& P, const HaloPlan& H, cons
 //     [unit - whole][cz][row of the chunk][position of the block] (forward_join_tail_kernel).
 // (few accumulators: four wavefronts per SIMD, i.e. at most 128 registers, also for the 512-thread
 // shape, so that two of its workgroups share a CU)
-// S: storage format of the tensors (see Store); with a 16-bit format T is float and csplit must be 1.
+// S: storage format of the tensors (see Store); T is float with a 16-bit format, and partial sums are always T.
 template <typename T, int ND, int MT, int NW, typename S = T>
 __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void forward_quad_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
                                                            const S* __restrict__ in,
                                                            const S* __restrict__ off, const S* __restrict__ Wq,
                                                            const S* __restrict__ bias, S* __restrict__ out,
-                                                           S* __restrict__ part, int csplit, unsigned whole) {
+                                                           T* __restrict__ part, int csplit, unsigned whole) {
     HaloPlan H;
     if (!chosen_halo(P, alts, sel, H)) return;          // another launch runs the chosen plan
     using MM = Mma<T>;
@@ -376,25 +376,29 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
 
     if (split && whole > 0) {
         // partial sums of a unit of the last round: [unit - whole][cz][MT * TN rows][NW * TN positions]
-        S* dst = part + ((size_t)(wg - whole) * csplit + cz) * (MT * TN) * (NW * TN) + wave * TN + j;
+        T* dst = part + ((size_t)(wg - whole) * csplit + cz) * (MT * TN) * (NW * TN) + wave * TN + j;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int r = 0; r < MM::NACC; ++r) dst[(size_t)(mt * TN + MM::row(r, q)) * (NW * TN)] = Store<S>::st(acc[mt][r]);
+            for (int r = 0; r < MM::NACC; ++r) dst[(size_t)(mt * TN + MM::row(r, q)) * (NW * TN)] = acc[mt][r];
         return;
     }
     if (!valid) return;
     // unsplit: the output with bias; every unit split: a partial output tensor per cz, the bias is added when they are joined
-    S* dst = split ? part + (size_t)cz * P.N * P.C_out * P.outV : out;
+    T* pdst = part + (size_t)cz * P.N * P.C_out * P.outV;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int r = 0; r < MM::NACC; ++r) {
             const int m = (mchunk * MT + mt) * TN + MM::row(r, q);
             if (m < P.M) {
+                const size_t at = ((size_t)n * P.C_out + g * P.M + m) * P.outV + pos;
                 T v = acc[mt][r];
-                if (bias && !split) v += Store<S>::ld(bias[g * P.M + m]);
-                dst[((size_t)n * P.C_out + g * P.M + m) * P.outV + pos] = Store<S>::st(v);
+                if (split) pdst[at] = v;
+                else {
+                    if (bias) v += Store<S>::ld(bias[g * P.M + m]);
+                    out[at] = Store<S>::st(v);
+                }
             }
         }
 }
@@ -403,10 +407,10 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
 // workgroup of NW * TN threads per unit and slice of JOIN_ROWS output channels, thread = position of
 // the block; out = bias + the csplit partial sums, added in the order of cz.
 constexpr int JOIN_ROWS = 8;
-template <typename T, int ND, int MT, int NW>
+template <typename T, int ND, int MT, int NW, typename S = T>
 __global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
-                                                                    const T* __restrict__ part, const T* __restrict__ bias,
-                                                                    T* __restrict__ out, int csplit, unsigned whole) {
+                                                                    const T* __restrict__ part, const S* __restrict__ bias,
+                                                                    S* __restrict__ out, int csplit, unsigned whole) {
     constexpr int TN = Mma<T>::TN, SLICES = MT * TN / JOIN_ROWS;
     static_assert(MT * TN % JOIN_ROWS == 0, "row slices");
     HaloPlan H;
@@ -435,7 +439,7 @@ __global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, Pl
 #pragma unroll
     for (int r = 0; r < JOIN_ROWS; ++r) {
         const int m = mchunk * MT * TN + (int)ml0 + r;
-        if (m < P.M) out[((size_t)tg_.n * P.C_out + g * P.M + m) * P.outV + pos] = bias ? v[r] + bias[g * P.M + m] : v[r];
+        if (m < P.M) out[((size_t)tg_.n * P.C_out + g * P.M + m) * P.outV + pos] = Store<S>::st(bias ? v[r] + (T)Store<S>::ld(bias[g * P.M + m]) : v[r]);
     }
 }
 

@@ -60,7 +60,9 @@ SETTINGS = [
     {"DCN_ADAPTIVE_MARGIN": "0", "DCN_FUSED_WAVES": "4", "DCN_FORWARD_WG": "512"},
 ]
 # the 16-bit forward through the float32 kernels: by request, and because the halo kernel declines the layer
-MIXED_SETTINGS = [{"DCN_NATIVE16": "0"}, {"DCN_HALO_MARGIN": "50"}, {"DCN_ADAPTIVE_MARGIN": "0"}]
+MIXED_SETTINGS = [{"DCN_NATIVE16": "0"}, {"DCN_HALO_MARGIN": "50"}, {"DCN_ADAPTIVE_MARGIN": "0"},
+                  # (the split last round of the 16-bit forward: float partial sums, rounded once when they are joined)
+                  {"DCN_FORWARD_SLOTS": "3"}, {"DCN_FORWARD_SLOTS": "5", "DCN_FORWARD_TAIL": "2"}]
 
 
 @pytest.mark.parametrize("extra", MIXED_SETTINGS, ids=lambda e: ",".join("%s=%s" % kv for kv in e.items()))
