@@ -1085,12 +1085,13 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     T* gout_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + ibytes);
     T* partial = reinterpret_cast<T*>(static_cast<char*>(ws) + ibytes + obytes);
     const dim3 tblock(32, 8);
-    hipLaunchKernelGGL(to_channels_last_kernel<T>, dim3((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N),
-                       tblock, 0, s, in, in_cl, P.C_in, P.inV);
-    if (int rc = check_launch("to_channels_last_kernel")) return rc;
-    hipLaunchKernelGGL(to_channels_last_kernel<T>, dim3((P.outV + 31) / 32, (unsigned)(P.C_out + 31) / 32, (unsigned)P.N),
-                       tblock, 0, s, gout, gout_cl, P.C_out, P.outV);
-    if (int rc = check_launch("to_channels_last_kernel")) return rc;
+    {
+        const unsigned vmax = P.inV > P.outV ? P.inV : P.outV;
+        const int cmax = P.C_in > P.C_out ? P.C_in : P.C_out;
+        hipLaunchKernelGGL(to_channels_last_pair_kernel<T>, dim3((vmax + 31) / 32, (unsigned)(cmax + 31) / 32, 2u * (unsigned)P.N), tblock, 0, s,
+                           in, in_cl, P.C_in, P.inV, gout, gout_cl, P.C_out, P.outV, P.N);
+        if (int rc = check_launch("to_channels_last_pair_kernel")) return rc;
+    }
     int rc;
     switch (MT) {
         case 1: rc = launch_bwd_weight<T, ND, 1>(P, in_cl, off, gout_cl, partial, s); break;
@@ -1099,7 +1100,7 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     }
     if (rc) return rc;
     const size_t rows_x_cg = (size_t)P.C_out * P.Cg, total = rows_x_cg * P.kV;
-    const unsigned rb = (unsigned)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+    const unsigned rb = (unsigned)((total + 63) / 64 > 8192 ? 8192 : (total + 63) / 64);
     hipLaunchKernelGGL(reduce_weight_partials_kernel<T>, dim3(rb), dim3(256), 0, s, partial, gw, P.nsplit, P.kV, rows_x_cg);
     return check_launch("reduce_weight_partials_kernel");
 }

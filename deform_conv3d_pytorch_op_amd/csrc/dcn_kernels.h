@@ -1624,15 +1624,62 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
 }
 
 // grad_weight[g*M+m][cl][tap] += sum over splits of partial[split][tap][g*M+m][cl]
+// 256 threads = 64 consecutive elements x 4 lanes of splits: lane l adds the splits l, l + 4, ...
+// (loads of a lane independent of each other), then the four sums are added in the order of l, so
+// the result does not depend on timing.
 template <typename T>
-__global__ void reduce_weight_partials_kernel(const T* __restrict__ partial, T* __restrict__ gw, int nsplit, int kV,
-                                              size_t rows_x_cg /* C_out * Cg */) {
+__global__ __launch_bounds__(256) void reduce_weight_partials_kernel(const T* __restrict__ partial, T* __restrict__ gw, int nsplit, int kV,
+                                                                     size_t rows_x_cg /* C_out * Cg */) {
+    __shared__ T part[4][64];
     const size_t total = (size_t)kV * rows_x_cg;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t tap = i / rows_x_cg, rc = i % rows_x_cg;         // rc = (g*M + m) * Cg + cl
+    const int e = threadIdx.x & 63, l = threadIdx.x >> 6;
+    for (size_t i0 = (size_t)blockIdx.x * 64; i0 < total; i0 += (size_t)gridDim.x * 64) {
+        const size_t i = i0 + e;
         T sum = 0;
-        for (int s = 0; s < nsplit; ++s) sum += partial[((size_t)s * kV + tap) * rows_x_cg + rc];
-        gw[rc * kV + tap] += sum;
+        if (i < total) {
+            const T* p = partial + i;
+            int s = l;
+            for (; s + 12 < nsplit; s += 16) {
+                const T a = p[(size_t)s * total], b = p[(size_t)(s + 4) * total], c = p[(size_t)(s + 8) * total], d = p[(size_t)(s + 12) * total];
+                sum += a; sum += b; sum += c; sum += d;
+            }
+            for (; s < nsplit; s += 4) sum += p[(size_t)s * total];
+        }
+        part[l][e] = sum;
+        __syncthreads();
+        if (l == 0 && i < total) {
+            const size_t tap = i / rows_x_cg, rc = i % rows_x_cg;     // rc = (g*M + m) * Cg + cl
+            gw[rc * kV + tap] += ((part[0][e] + part[1][e]) + part[2][e]) + part[3][e];
+        }
+        __syncthreads();
+    }
+}
+
+// Both layout changes of backward_weight in one launch: z < N copies tensor A, z >= N tensor B
+// (grid: the larger of the two extents along x and y, 2 * N along z).
+template <typename T>
+__global__ void to_channels_last_pair_kernel(const T* __restrict__ srcA, T* __restrict__ dstA, int CA, unsigned VA,
+                                             const T* __restrict__ srcB, T* __restrict__ dstB, int CB, unsigned VB, int N) {
+    __shared__ T tile[32][33];
+    const bool second = (int)blockIdx.z >= N;
+    const T* src = second ? srcB : srcA;
+    T* dst = second ? dstB : dstA;
+    const int C = second ? CB : CA;
+    const unsigned V = second ? VB : VA;
+    const unsigned v0 = blockIdx.x * 32;
+    const int c0 = blockIdx.y * 32;
+    if (v0 >= V || c0 >= C) return;                 // uniform for the block
+    const size_t base = (size_t)(second ? blockIdx.z - N : blockIdx.z) * C * V;
+    for (int i = threadIdx.y; i < 32; i += 8) {
+        const int c = c0 + i;
+        const unsigned v = v0 + threadIdx.x;
+        if (c < C && v < V) tile[i][threadIdx.x] = src[base + (size_t)c * V + v];
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += 8) {
+        const unsigned v = v0 + i;
+        const int c = c0 + threadIdx.x;
+        if (c < C && v < V) dst[base + (size_t)v * C + c] = tile[threadIdx.x][i];
     }
 }
 
