@@ -103,7 +103,9 @@ def run_config(name, a):
     spec = CONFIGS[name]
     dtype = getattr(torch, spec[-1])
     kw = dict(dtype=dtype, seed=0, bias=False)
-    if spec[-2] == "normal_mix":
+    if a.offset_scale is not None:      # not the configuration's own offsets: U[-s, s]
+        c = make_case(*spec[:-2], a.offset_scale, **kw)
+    elif spec[-2] == "normal_mix":
         c = make_case(*spec[:-2], 1.0, off_dist="normal_mix", **kw)
     else:
         c = make_case(*spec[:-1], **kw)
@@ -196,7 +198,7 @@ def run_config(name, a):
     achieved = F / (kernel_ms[dominant] * 1e-3) / 1e12
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": round(achieved, 3), "peak": peak,
                 "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                "traffic": measured_traffic(name, dominant),
+                "traffic": measured_traffic(name, dominant) if a.offset_scale is None else None,
                 "ms": round(kernel_ms[dominant], 4),
                 "algorithmic_flops": F, "algorithmic_bytes": ab[dominant],
                 "hbm_frac_at_algorithmic_bytes": round(ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
@@ -237,7 +239,8 @@ def run_config(name, a):
         "ms_per_step": round(ms_step, 4), "fwd_ms": round(ms_fwd, 4),
         "ms_per_step_events": step_events, "fwd_ms_events": fwd_events, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32" if dtype == torch.float32 else "f64", "data": "synthetic",
-        "config": {"workload": name + ": " + DESCR[name]},
+        "config": {"workload": name + ": " + DESCR[name] +
+                               ("" if a.offset_scale is None else " -- with offsets U[-%g,%g] instead of its own" % (a.offset_scale, a.offset_scale))},
         "mfma_frac_whole_step": round(value / peak, 4),
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
     }
@@ -250,6 +253,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c4", choices=sorted(CONFIGS) + ["all"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--offset-scale", type=float, default=None,
+                    help="offsets uniform in [-s, s] instead of the configuration's own (how the rates depend on the reach of the offsets)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic for scaling rocprof's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
