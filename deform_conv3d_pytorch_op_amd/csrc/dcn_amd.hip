@@ -73,7 +73,9 @@ template <typename T> size_t bwd_data_weight_bytes(int M, int Cg, int kV, int G,
     const size_t C_in = (size_t)Cg * G;
     const size_t packed4 = packed_weight_elems<T>(M, kV, slab_bound(C_in, G, cpg, 4), 4);
     const size_t packed8 = packed_weight_elems<T>(M, kV, slab_bound(C_in, G, cpg, 8), 8);
-    const size_t packed = packed4 > packed8 ? packed4 : packed8;
+    const size_t packed16 = packed_weight_elems<T>(M, kV, slab_bound(C_in, G, cpg, 16), 16);
+    size_t packed = packed4 > packed8 ? packed4 : packed8;
+    if (packed16 > packed) packed = packed16;
     return align256((plain > packed ? plain : packed) * sizeof(T));
 }
 // Partial outputs of a forward pass that splits the input channels of a position block over several
@@ -188,7 +190,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
 //   DCN_COORD=separate     grad_offset from the channels-last kernel instead of the fused LDS-halo kernel
 //   DCN_FUSED_WAVES=4      fused backward kernel with four wavefronts per workgroup even where eight fit
-//   DCN_FUSED_CHUNK=4      fused backward kernel with 4-channel chunks also where it would take 8 (2-D layers)
+//   DCN_FUSED_CHUNK=4      fused backward kernel with 4-channel chunks also where it would take 8 or 16; =8: never 16 (2-D layers)
 //   DCN_FUSED_TAIL=0       fused backward kernel: all items split alike, never only those of the last round
 //   DCN_CSPLIT=n           fused backward kernel: every item split over n workgroups
 //   DCN_FUSED_SLOTS=n      fused backward kernel: plan the launch as if n workgroups ran at once (test hook)
@@ -244,6 +246,10 @@ static int wide_forward() {      // 0 never, 1 when it pays, 2 whenever the halo
         return !e ? 1 : atoi(e) == 512 ? 0 : atoi(e) == 1024 ? 2 : 1;
     }();
     return v;
+}
+static bool fused_chunk16() {     // DCN_FUSED_CHUNK=8 (or 4): never take 16-channel chunks in the fused backward kernel
+    static const int v = [] { const char* e = getenv("DCN_FUSED_CHUNK"); return (e && (atoi(e) == 8 || atoi(e) == 4)) ? 0 : 1; }();
+    return v != 0;
 }
 static bool fused_chunk8() {      // DCN_FUSED_CHUNK=4: never take 8-channel chunks in the fused backward kernel
     static const int v = [] { const char* e = getenv("DCN_FUSED_CHUNK"); return (e && atoi(e) == 4) ? 0 : 1; }();
@@ -756,16 +762,20 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             auto passes = [&](int c) { const int tp = Mma<T>::TN / c; return (P.kV + tp - 1) / tp; };
             const bool eight = (ND == 2 || pair) && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
                                (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 8;
-            const int cch = eight ? 8 : 4;
+            // 16 (2-D, float, paired cells): two taps per pass -- the 9 taps of a 3x3 kernel are 5 passes per 16
+            // channels instead of 6
+            const bool sixteen = ND == 2 && pair && eight && fused_chunk16() && seg >= 16 && passes(16) * 8 < passes(8) * 16 &&
+                                 (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 16;
+            const int cch = sixteen ? 16 : eight ? 8 : 4;
             Ph.cchunk = cch;
             if (fixed && !eight) Ph.hstride = FUSED_HS;
             const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
             // grad_output operand held in registers when its reduction steps fit: 32 per pass
             // (M <= 64 float, 128 double with 4-channel chunks)
             const int ksteps = (P.M + Mma<T>::KL - 1) / Mma<T>::KL;
-            const bool wide = eight && pair && ksteps <= 32;                                         // the kernel's WIDE
-            const int slot_regs = wide ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
-            const bool breg = ksteps <= Mma<T>::NACC / slot_regs * (wide ? 16 : 8);
+            const bool wide = eight && !sixteen && pair && ksteps <= 32;                             // the kernel's WIDE
+            const int slot_regs = (wide || sixteen) ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
+            const bool breg = ksteps <= Mma<T>::NACC / slot_regs * ((wide || sixteen) ? 16 : 8);
             // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
             const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
             Kern kern = nullptr;
@@ -773,7 +783,9 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
 #define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2>
             auto pick = [&](auto pair_tag) {
                 constexpr bool PR = decltype(pair_tag)::value;
-                if (eight) {
+                if (sixteen) {
+                    if constexpr (ND == 2 && PR && sizeof(T) == 4) kern = breg ? DCN_FUSED_C(16, true, 0, 8, PR) : DCN_FUSED_C(16, false, 0, 8, PR);
+                } else if (eight) {
                     if constexpr (ND == 2 || PR) kern = breg ? DCN_FUSED_C(8, true, 0, 8, PR) : DCN_FUSED_C(8, false, 0, 8, PR);
                 } else if (breg2) {
                     if constexpr (sizeof(T) == 4) {
@@ -874,9 +886,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             bool packed = false;
             for (int e = 0; e < k; ++e) packed = packed || fp[e].wt == fp[k].wt;
             if (packed) continue;
-            const bool eight = fp[k].cch == 8, wide = fp[k].wide;
-            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)(eight ? chunk_candidates<8>(P.cpg, P.Cg, P.C_in)
-                                                                                      : chunk_candidates<4>(P.cpg, P.Cg, P.C_in)), fp[k].cch);
+            const bool sixteen = fp[k].cch == 16, eight = fp[k].cch == 8, wide = fp[k].wide;
+            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)(sixteen ? chunk_candidates<16>(P.cpg, P.Cg, P.C_in)
+                                                                            : eight ? chunk_candidates<8>(P.cpg, P.Cg, P.C_in)
+                                                                                    : chunk_candidates<4>(P.cpg, P.Cg, P.C_in)), fp[k].cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
             PlanChoice pk = pc;
             if (k > 0) pk.sel = nullptr;
@@ -884,7 +897,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             T* dst = const_cast<T*>(fp[k].wt);
             const dim3 pgrid(blocks + (pk.sel ? 1 : 0));
             // (wide: row order that leaves the eight channels of a tap in one lane)
-            if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            if (sixteen) hipLaunchKernelGGL((pack_weight_kernel<T, 16>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            else if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
             else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
             else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
             if (int rc = check_launch("pack_weight_kernel")) return rc;

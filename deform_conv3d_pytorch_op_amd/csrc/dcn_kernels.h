@@ -798,6 +798,10 @@ __global__ __launch_bounds__(512) void weight_bounds_kernel(const T* __restrict_
 // of a channel becomes an immediate offset of the LDS instructions instead of address arithmetic.
 // PACKW: the weights come in the per-chunk lane order of pack_weight_kernel instead of
 // [g][tap][m][channel].
+// CCH = 16 (float, 2-D layers whose halo leaves room for 16 channel planes): two taps per pass, so the
+// nine taps of a 3x3 kernel take 5 passes per 16 channels instead of 6, with half as many chunks to
+// zero, stage and flush; a lane then holds eight channels of each of the two taps (0..3 and 8..11 in
+// lane group 0, 4..7 and 12..15 in lane group 1) and walks them as two tap slots.
 // PAIR (float only): the cells hold two channels each as 32-bit fixed point (LdsCell<float>::add2):
 // half the LDS atomics and two thirds of the LDS bytes per channel.  The terms are scaled such
 // that (positions of the block x taps) of the largest possible one -- all that a cell can receive
@@ -823,7 +827,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     // channels of each of four taps, with the other four in the other lane group: the geometry of a
     // (tap, position) is then worked out once per eight channels, not once per lane group.
     constexpr bool WIDE = PAIR && CCH == 8 && BREG;      // (with the grad_output operand in registers: measured slower without)
-    constexpr int RPS = WIDE ? 8 : (MM::row(1, 0) - MM::row(0, 0) == 1) ? 4 : CCH / 4;   // registers that share a tap
+    // (16-channel chunks, float: two taps per pass, a lane holds eight channels of each -- 0..3 and 8..11 or 4..7 and 12..15)
+    constexpr int RPS = (WIDE || CCH == 16) ? 8 : (MM::row(1, 0) - MM::row(0, 0) == 1) ? 4 : CCH / 4;   // registers that share a tap
     constexpr int NS = NACC / RPS;                      // tap slots per lane and pass
     // (tap of the pass, channel of the chunk) behind accumulator register r of lane group qq
     auto row_tap = [](int r, int qq) { return WIDE ? 2 * (r / 8) + qq : MM::row(r, qq) / CCH; };
@@ -885,7 +890,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
         // wave-uniform base (scalar registers) + 32-bit lane offset of the B operand grad_output[m][pos]
-        constexpr int AB = WIDE ? 16 : 8;           // reduction steps per operand batch (NS * AB = 32 ride on a pass)
+        constexpr int AB = (WIDE || CCH == 16) ? 16 : 8;      // reduction steps per operand batch (NS * AB = 32 ride on a pass)
         const T* gbase = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV;
         const unsigned b_off = (unsigned)q * P.outV + pos;
         const size_t gstep = (size_t)KL * P.outV;

@@ -10,7 +10,8 @@ settings, each in a process of its own (the knobs are read once per process):
   DCN_COORD=separate   grad_offset from the channels-last kernel, grad_input from the scatter-only kernel
   DCN_CSPLIT=1 / 4     channel chunks of the fused backward kernel on one / four workgroups
   DCN_FUSED_WAVES=4    the fused backward kernel's four-wavefront shape (otherwise only strided full-size cases use it)
-  DCN_FUSED_CHUNK=4    the fused backward kernel with 4-channel chunks also for 2-D layers (which otherwise take 8)
+  DCN_FUSED_CHUNK=4    the fused backward kernel with 4-channel chunks also for 2-D layers (which otherwise take 16, or 8
+                       where a deformable group has fewer than 16 channels); =8: 8-channel chunks where it would take 16
   DCN_FUSED_SLOTS=3    plans the fused backward launch for a device of three workgroups: unsplit items first, the
                        items of the last round split over several workgroups (otherwise only full-size layers get there)
   DCN_FUSED_TAIL=0     ... and the same without that split; DCN_FUSED_FIXED=0: runtime plane stride
@@ -45,6 +46,7 @@ SETTINGS = [
     {"DCN_COORD": "separate"},
     {"DCN_FUSED_WAVES": "4"},
     {"DCN_FUSED_CHUNK": "4"},
+    {"DCN_FUSED_CHUNK": "8"},
     {"DCN_FUSED_SLOTS": "3"},
     {"DCN_FUSED_SLOTS": "3", "DCN_FUSED_TAIL": "0", "DCN_FUSED_FIXED": "0"},
     {"DCN_OVERLAP_BACKWARD": "1", "DCN_FORWARD_SPLIT": "0"},
