@@ -65,6 +65,9 @@ SMALL_CASES = {
     "2d_k7": (2, 1, 8, 10, (12, 11), 7, 1, 3, 1, 8, 1, 2.0),                   # 49 taps
     "3d_m72_chunk8": (3, 1, 16, 72, (4, 8, 9), 3, 1, 1, 1, 8, 1, 1.5),        # 36 reduction steps: the grad_output operand does not fit the registers
     "3d_m100_chunk4": (3, 1, 8, 100, (4, 8, 9), 3, 1, 1, 1, 4, 1, 1.5),       # 50 reduction steps, 4-channel chunks: the operand takes two register sets
+    "2d_chunk16_small_m": (2, 1, 32, 24, (12, 13), 3, 1, 1, 1, 16, 1, 1.5),    # 16-channel chunks (float32), grad_output operand in registers, two deformable groups
+    "2d_chunk16_ragged": (2, 2, 44, 100, (10, 9), 3, 1, 1, 1, 22, 1, 2.0),     # 22-channel segments: chunks of 16 + 6, 50 reduction steps
+    "2d_chunk16_k1": (2, 1, 16, 8, (9, 10), 1, 1, 0, 1, 16, 1, 1.0),           # a single tap: one pass of two tap slots, one of them empty
 }
 
 
