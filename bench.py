@@ -98,7 +98,7 @@ def run_config(name, a):
     import deform_conv3d_pytorch_op_amd as dcn
     from deform_conv3d_pytorch_op_amd import _lib
     from deform_conv3d_pytorch_op_amd.functions import _geom
-    from tests.cases import make_case
+    from deform_conv3d_pytorch_op_amd.synthetic import make_case
 
     spec = CONFIGS[name]
     dtype = getattr(torch, spec[-1])

@@ -811,9 +811,8 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             // the items of the whole rounds stay unsplit and only those of the last round are split, as
             // finely as fills the device; they come last in the launch.  A workgroup's fixed part
             // (grad_output operand, halo table, offsets) costs about a quarter of a chunk, which the
-            // estimate charges per split.  The chunks of an item add their grad_offset parts with float
-            // atomics on a zero-filled buffer (measured faster than read-modify-write by one workgroup);
-            // an item of a single chunk stores.
+            // estimate charges per split.  The workgroups that share an item add their grad_offset parts with
+            // float atomics on a zero-filled buffer; the only owner of an item stores running sums.
             const int nchunks = (seg + cch - 1) / cch;
             const long long items = (long long)Ph.N * Ph.tiles * Ph.DG;
             const long long slots = forced_slots() ? forced_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
@@ -836,7 +835,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (forced_csplit()) { csplit = forced_csplit(); whole = 0; }
             if (csplit > nchunks) csplit = nchunks;
             if (whole + (items - whole) * csplit > 0x7fffffffLL) continue;
-            fp.Ph = Ph; fp.kern = kern; fp.nw = nw; fp.cch = cch; fp.csplit = csplit; fp.goff_atomic = nchunks > 1 ? 1 : 0;
+            fp.Ph = Ph; fp.kern = kern; fp.nw = nw; fp.cch = cch; fp.csplit = csplit; fp.goff_atomic = csplit > 1 ? 1 : 0;
             fp.wide = wide; fp.whole = whole; fp.items = items; fp.slots = slots; fp.lds = lds; fp.wt = nullptr;
             return true;
         }
@@ -1086,6 +1085,8 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
     if (!in || !off || !gout || !gw) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     if (int rc = device_info(nullptr)) return rc;
     if ((long long)P.outV * P.C_out > (1ll << 31)) return fail(DCN_E_ARGUMENT, "one output sample exceeds 2^31 elements");
+    // (the layout change of both operands is one launch with 2 * N slices along z)
+    if (2 * (long long)P.N > 65535) return fail(DCN_E_ARGUMENT, "backward_weight: batch exceeds 32767");
     // the kernel addresses both operands by 32-bit byte offsets from the sample's base
     if ((unsigned long long)P.inV * P.C_in * sizeof(T) >= (1ull << 32) || (unsigned long long)P.outV * P.C_out * sizeof(T) >= (1ull << 32))
         return fail(DCN_E_ARGUMENT, "one sample of the input or of grad_output reaches 4 GiB");

@@ -848,9 +848,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     // Work items are (tile, deformable group) pairs.  The first `whole` workgroups of the launch take
     // one item each; every later item is shared by csplit workgroups, of which workgroup cz takes
     // every csplit-th channel chunk: finer work at the end of the launch fills the last, ragged
-    // round of workgroups.  goff_atomic: the grad_offset contributions of the channel chunks meet
-    // through float atomics on a zero-filled buffer (required where an item is shared); otherwise
-    // the first chunk stores and later ones add in place.
+    // round of workgroups.  The grad_offset contributions of the channel chunks of a shared item meet
+    // through float atomics on a zero-filled buffer (the host passes goff_atomic = 1 when the launch
+    // has shared items and has cleared the buffer); the single owner of an item stores the first
+    // chunk's values and then the running sum.
     unsigned item;
     int cz = 0, cs = 1;
     if (blockIdx.x < whole) item = xcd_contiguous(blockIdx.x, whole);
@@ -862,6 +863,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     }
     const unsigned nt = (unsigned)P.N * P.tiles;
     const int dg = item / nt;
+    // an item that several workgroups share needs the atomics (the host has zero-filled grad_offset);
+    // the only owner of an item stores the running sum over its chunks instead
+    goff_atomic = cs > 1 ? 1 : 0;
 
     TileGeo<ND> tg;
     tile_decode<ND>(P, H, item % nt, tg);
@@ -1089,6 +1093,13 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             // that swap roles from slot to slot (NS is even): copying "next" into "current" would have
             // to wait for the loads at the copy, a whole slot before the values are needed
             T o_buf[2][ND], kd_buf[2][ND];
+            // grad_offset of an item that one workgroup owns alone: what the earlier chunks have written
+            // for the slot's (tap, position) travels with the slot's offsets and the sum is stored --
+            // plain loads and stores that stay in the L2 between two chunks, where float atomics are
+            // limited to about one per clock and L2 channel (130 M of them per call on a 64-channel
+            // 3x3x3 layer of 200 k positions)
+            T p_buf[2][ND];
+            const bool rmw_prev = COORD && !goff_atomic && !first_chunk;        // uniform
             static_assert(NS % 2 == 0, "offset buffers alternate within a pass");
             // Kernel coordinates of this lane's tap in the next slot, counted up with the slots (the
             // taps of consecutive slots are TP / NS apart for every lane).  They live in registers: a
@@ -1110,6 +1121,13 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 const T* ob = off_dg + (size_t)tu * ND * P.outV;
 #pragma unroll
                 for (int a = 0; a < ND; ++a) o_nx[a] = (ob + (size_t)a * P.outV)[lo];
+                if constexpr (COORD) {
+                    if (rmw_prev) {
+                        const T* gb = goff_dg + (size_t)tu * ND * P.outV;
+#pragma unroll
+                        for (int a = 0; a < ND; ++a) p_buf[ts & 1][a] = (gb + (size_t)a * P.outV)[lo];
+                    }
+                }
 #pragma unroll
                 for (int a = 0; a < ND; ++a) kd_nx[a] = (T)(kq[a] * P.dil[slot<ND>(a)]);
 #pragma unroll
@@ -1139,8 +1157,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                     for (int a = 0; a < ND; ++a) {
                         if (goff_atomic) { if (pend_ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, pend_ga[a]); }
-                        else if (first_chunk) gp[(size_t)a * P.outV] = pend_ga[a];
-                        else gp[(size_t)a * P.outV] += pend_ga[a];
+                        else gp[(size_t)a * P.outV] = pend_ga[a];       // (the earlier chunks' sum is part of it)
                     }
                 }
                 pend = false;
@@ -1393,7 +1410,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         pend = slot_ok && owner;
                         pend_tap = tap;
 #pragma unroll
-                        for (int a = 0; a < ND; ++a) pend_ga[a] = ga[a];
+                        for (int a = 0; a < ND; ++a) pend_ga[a] = rmw_prev ? ga[a] + p_buf[ts & 1][a] : ga[a];
                     }
                     __builtin_amdgcn_sched_barrier(0);      // one tap slot at a time: keeps the live register set small
                 }

@@ -55,7 +55,7 @@ extern "C" {
 #define DCN_E_ARGUMENT   -1   /* inconsistent extents, null pointer, unsupported size */
 #define DCN_E_WORKSPACE  -2   /* workspace missing or too small */
 #define DCN_E_LAUNCH     -3   /* HIP reported an error when launching */
-#define DCN_E_DEVICE     -4   /* no current HIP device, or a query of it failed */
+#define DCN_E_DEVICE     -4   /* no current HIP device, a query of it failed, or it is not a gfx950 GPU */
 
 int dcn_version(void);              /* ABI version, currently 1 */
 const char *dcn_arch(void);         /* the code-object target the kernels were built for: "gfx950" */

@@ -30,12 +30,20 @@ def _both(L, spec, seed, poison):
     stream = torch.cuda.current_stream().cuda_stream
     _lib.check(L.dcn3d_forward_f32(x.data_ptr(), w.data_ptr(), off.data_ptr(), b.data_ptr(), want.data_ptr(), *geom,
                                    ws.data_ptr(), ws_bytes, stream))
+    # a first call resolves the scratch array's device address (once per device); the call that is
+    # checked for allocations comes after it
+    _lib.check(L.dcn3d_forward_noalloc_f32(x.data_ptr(), w.data_ptr(), off.data_ptr(), b.data_ptr(), got.data_ptr(),
+                                           *geom, stream))
+    torch.cuda.synchronize()
+    got.fill_(poison)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated(dev)
+    free_before = torch.cuda.mem_get_info(dev)[0]       # the driver's free bytes: sees allocations made behind torch's back
     _lib.check(L.dcn3d_forward_noalloc_f32(x.data_ptr(), w.data_ptr(), off.data_ptr(), b.data_ptr(), got.data_ptr(),
                                            *geom, stream))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
     return got, want
 
 
