@@ -332,7 +332,7 @@ static int forced_csplit() {    // DCN_CSPLIT=n: workgroups per (tile, deformabl
 
 template <typename T, int ND>
 bool plan_halo(Params& P, size_t budget, int m, int max_chunk = 1 << 30, size_t cell_bytes = sizeof(T), int waves = WAVESH,
-               bool smallest_halo = false, int chunk_mult = 0, const int* blocks = nullptr) {
+               bool smallest_halo = false, int chunk_mult = 0, const int* blocks = nullptr, int wmult = 1) {
     const int npos = waves * Mma<T>::TN;        // positions per workgroup, one column tile per wavefront
     int td[3] = {1, 1, 1};
     if (ND == 3) { td[1] = 8; td[2] = 8; td[0] = npos / 64; }
@@ -361,6 +361,9 @@ bool plan_halo(Params& P, size_t budget, int m, int max_chunk = 1 << 30, size_t 
         P.mlo[a] = used ? m : 0;
         // lowest corner: base - m; highest corner: base + m (the high corner of a sample at base + m - eps)
         P.hext[a] = used ? (td[a] - 1) * P.stride[a] + (P.k[a] - 1) * P.dil[a] + 1 + 2 * m : 1;
+        // (wmult: the innermost extent rounded up to a multiple, for kernels whose LDS layout depends on
+        // the position of a halo voxel modulo that number; the extra cells lie on the high side)
+        if (a == 2 && wmult > 1) P.hext[a] = (P.hext[a] + wmult - 1) / wmult * wmult;
         hvol *= P.hext[a];
         tiles *= P.ntile[a];
     }
@@ -727,11 +730,13 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     // Eight wavefronts per workgroup; four (half the positions, in the block shape with the smallest
     // halo) where only that fits, e.g. under stride 2.
     constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
+    constexpr int FUSED_HS8 = 2016;     // plane stride of the 8-channel float instantiation with compile-time halo extents
     using Kern = void (*)(Params, PlanSet, const unsigned*, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
     struct FusedPlan {
         Params Ph;
         Kern kern;
         int nw, cch, csplit, goff_atomic;
+        bool zero_goff;
         bool wide;
         long long whole, items, slots;
         size_t lds;
@@ -750,26 +755,40 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             // (positions of the block x taps) leave at least 17 bits below the largest possible term
             const bool pair = sizeof(T) == 4 && fused_pair() && (long long)nw * TN * P.kV <= (1 << 14);
             const size_t chb = (pair ? 4 : 8) + sizeof(T);      // LDS bytes per channel and halo voxel: cell + input value
-            if (!plan_halo<T, ND>(Ph, scatter_budget(), m, 8, chb, nw, smallest)) continue;
-            const size_t tables = (size_t)Ph.hvol * 4;      // halo table
-            const bool fixed = fused_fixed_stride() && Ph.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * chb + tables <= scatter_budget();
-            if ((long long)Ph.N * Ph.tiles * Ph.DG * 4 > 0x7fffffffLL) continue;
-            if (!fixed && (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) < 4) continue;
             // Channels per chunk: 8 where that takes fewer MFMA passes per channel (a pass holds TN / CCH
             // taps: the 9 taps of a 3x3 kernel are 2 float passes per 4 channels or 3 per 8; the 27 of a
             // 3x3x3 kernel 4 or 7) and the planes of 8 channels fit: the small halos of 2-D layers, and
-            // 3-D ones with paired cells.
+            // 3-D ones with paired cells.  16 (2-D, float, paired cells): two taps per pass -- the 9 taps of
+            // a 3x3 kernel are 5 passes per 16 channels instead of 6.  The float kernel with 8 channels
+            // per chunk keeps the input values bank-swizzled and wants the innermost halo extent a
+            // multiple of the four-channel groups per voxel.
             auto passes = [&](int c) { const int tp = Mma<T>::TN / c; return (P.kV + tp - 1) / tp; };
-            const bool eight = (ND == 2 || pair) && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8 &&
-                               (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 8;
-            // 16 (2-D, float, paired cells): two taps per pass -- the 9 taps of a 3x3 kernel are 5 passes per 16
-            // channels instead of 6
-            const bool sixteen = ND == 2 && pair && eight && fused_chunk16() && seg >= 16 && passes(16) * 8 < passes(8) * 16 &&
-                                 (scatter_budget() - tables) / ((size_t)Ph.hstride * chb) >= 16;
-            const int cch = sixteen ? 16 : eight ? 8 : 4;
+            int cch = 0;
+            size_t tables = 0;
+            bool fixed = false, special = false;
+            for (int cand = 16; cand >= 4 && !cch; cand /= 2) {
+                if (cand >= 8 && !((ND == 2 || pair) && nw == 8 && fused_chunk8() && seg >= 8 && passes(8) * 4 < passes(4) * 8)) continue;
+                if (cand == 16 && !(ND == 2 && pair && fused_chunk16() && seg >= 16 && passes(16) * 8 < passes(8) * 16)) continue;
+                Params Pc = P;
+                const int wmult = cand == 16 ? 1 : cand == 8 ? swizzle_groups<T, 8>() : 1;
+                if (!plan_halo<T, ND>(Pc, scatter_budget(), m, 8, chb, nw, smallest, 0, nullptr, wmult)) continue;
+                const size_t tb = (size_t)Pc.hvol * 4;      // halo table
+                if ((long long)Pc.N * Pc.tiles * Pc.DG * 4 > 0x7fffffffLL) continue;
+                if (cand >= 8) {
+                    if ((scatter_budget() - tb) / ((size_t)Pc.hstride * chb) < (size_t)cand) continue;
+                } else {
+                    // A halo of up to FUSED_HS cells gets the variant with that compile-time plane stride
+                    fixed = fused_fixed_stride() && Pc.hvol <= FUSED_HS && (size_t)4 * FUSED_HS * chb + tb <= scatter_budget();
+                    if (!fixed && (scatter_budget() - tb) / ((size_t)Pc.hstride * chb) < 4) continue;
+                }
+                Ph = Pc;
+                tables = tb;
+                cch = cand;
+            }
+            if (!cch) continue;
+            const bool sixteen = cch == 16, eight = cch >= 8;
             Ph.cchunk = cch;
             if (fixed && !eight) Ph.hstride = FUSED_HS;
-            const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
             // grad_output operand held in registers when its reduction steps fit: 32 per pass
             // (M <= 64 float, 128 double with 4-channel chunks)
             const int ksteps = (P.M + Mma<T>::KL - 1) / Mma<T>::KL;
@@ -778,6 +797,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             const bool breg = ksteps <= Mma<T>::NACC / slot_regs * ((wide || sixteen) ? 16 : 8);
             // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
             const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
+            special = ND == 3 && eight && !sixteen && pair && wide && breg && fused_fixed_stride() && Ph.hext[1] == 14 && Ph.hext[2] == 14 &&
+                      Ph.hstride <= FUSED_HS8;
+            if (special) Ph.hstride = FUSED_HS8;
+            const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
             Kern kern = nullptr;
 #define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>
 #define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2>
@@ -787,6 +810,11 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
                     if constexpr (ND == 2 && PR && sizeof(T) == 4) kern = breg ? DCN_FUSED_C(16, true, 0, 8, PR) : DCN_FUSED_C(16, false, 0, 8, PR);
                 } else if (eight) {
                     if constexpr (ND == 2 || PR) kern = breg ? DCN_FUSED_C(8, true, 0, 8, PR) : DCN_FUSED_C(8, false, 0, 8, PR);
+                    // the halo of a 3x3x3 kernel at stride 1 and margin 2 under the default block of positions:
+                    // inner extents 14 x 14 and the plane stride fixed at compile time
+                    if constexpr (ND == 3 && PR && sizeof(T) == 4) {
+                        if (special) kern = backward_input_halo_kernel<T, ND, 8, true, true, FUSED_HS8, 8, true, true, 1, 14, 14>;
+                    }
                 } else if (breg2) {
                     if constexpr (sizeof(T) == 4) {
                         if (nw == 8) kern = fixed ? DCN_FUSED_B2(FUSED_HS, 8, PR) : DCN_FUSED_B2(0, 8, PR);
@@ -835,7 +863,12 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (forced_csplit()) { csplit = forced_csplit(); whole = 0; }
             if (csplit > nchunks) csplit = nchunks;
             if (whole + (items - whole) * csplit > 0x7fffffffLL) continue;
-            fp.Ph = Ph; fp.kern = kern; fp.nw = nw; fp.cch = cch; fp.csplit = csplit; fp.goff_atomic = csplit > 1 ? 1 : 0;
+            fp.Ph = Ph; fp.kern = kern; fp.nw = nw; fp.cch = cch; fp.csplit = csplit;
+            // grad_offset over the chunks of an item that one workgroup owns: the running sum through plain
+            // loads and stores in the 3-D kernels (float atomics run at about 3e11 per second over the device,
+            // and a 3x3x3 layer has 81 grad_offset elements per position and chunk); atomics in the 2-D ones
+            fp.goff_atomic = ND == 2 && nchunks > 1 ? 1 : 0;
+            fp.zero_goff = fp.goff_atomic || csplit > 1;
             fp.wide = wide; fp.whole = whole; fp.items = items; fp.slots = slots; fp.lds = lds; fp.wt = nullptr;
             return true;
         }
@@ -904,7 +937,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         }
         if (int rc = weight_bounds<T>(P, w, wmax, s)) return rc;
         bool any_atomic = false;
-        for (int k = 0; k < pc.nplans; ++k) any_atomic = any_atomic || fp[k].goff_atomic;
+        for (int k = 0; k < pc.nplans; ++k) any_atomic = any_atomic || fp[k].zero_goff;
         if (any_atomic) {
             const size_t nel = (size_t)P.N * P.DG * P.kV * ND * P.outV;
             const unsigned fb = (unsigned)((nel + 1023) / 1024 > 8192 ? 8192 : (nel + 1023) / 1024);

@@ -13,6 +13,7 @@
 // voxel in 16 (32) consecutive bytes, one wide LDS read per corner fetches all of them, and the
 // interpolated values of the four channels are the B operands of four MFMA steps.
 #pragma once
+#include <limits>
 #include "dcn_kernels.h"
 
 #include <type_traits>
@@ -99,8 +100,9 @@ __global__ void pack_forward_weight_kernel(Params P, const S* __restrict__ W, S*
 // the latter with weight zero).
 template <typename T, int WGS, typename S = T>
 __device__ inline void halo_stage_quads(const Params& P, const HaloPlan& H, const S* __restrict__ chan0, int nch,
-                                        const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
+                                        const unsigned* __restrict__ sTab, T* __restrict__ sIn, int* __restrict__ nonfinite) {
     const int ngrp = (nch + FQ - 1) / FQ;
+    bool bad = false;                  // a NaN or an infinity among the staged values (see halo_nonfinite)
     for (int v = threadIdx.x; v < H.hvol; v += WGS) {
         const unsigned t = sTab[v];
         const unsigned g = t == ~0u ? 0u : t;
@@ -109,10 +111,13 @@ __device__ inline void halo_stage_quads(const Params& P, const HaloPlan& H, cons
 #pragma unroll
             for (int e = 0; e < FQ; ++e) val[e] = Store<S>::ld(chan0[(size_t)min(grp * FQ + e, nch - 1) * P.inV + g]);
 #pragma unroll
+            for (int e = 0; e < FQ; ++e) bad = bad || !(fabs(val[e]) <= std::numeric_limits<T>::max());
+#pragma unroll
             for (int e = 0; e < FQ; ++e)
                 sIn[((size_t)grp * H.hstride + v) * FQ + e] = (grp * FQ + e < nch && t != ~0u) ? val[e] : (T)0;
         }
     }
+    if (bad) *nonfinite = 1;
 }
 
 // 1-D grid of N * tiles (blocks of positions) * G * mchunks * csplit workgroups of NW wavefronts;
@@ -143,6 +148,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     constexpr bool S16 = sizeof(S) == 2;                // 16-bit storage: 16-bit matrix instructions
     typedef T V4 __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    __shared__ int sNonFinite;
     T* sIn = reinterpret_cast<T*>(smem_raw);                                            // [cchunk / 4][hstride][4]
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (size_t)H.cchunk * H.hstride);   // [hvol]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -202,9 +208,16 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
             const int nch = min(H.cchunk, ce - cc0);
             const int ngrp = (nch + FQ - 1) / FQ;
             const S* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
+            if (threadIdx.x == 0) sNonFinite = 0;
             __syncthreads();                                               // readers of the previous chunk are done
-            halo_stage_quads<T, WGS, S>(P, H, chan0, nch, sTab, sIn);
+            halo_stage_quads<T, WGS, S>(P, H, chan0, nch, sTab, sIn, &sNonFinite);
             __syncthreads();
+            // Non-finite input values in this halo: the branch-free sampler reads the cell next to a
+            // collapsed corner with weight 0, and 0 * inf would be NaN where the reference never
+            // touches that voxel (deform3d/lib/deform_conv3d_cuda_kernel.cu:24-26).  Samples in the
+            // collapse zones (p <= 0 or p >= size - 1 on some axis) then take the pass through global
+            // memory, which follows the reference's corner rule.
+            const bool halo_nonfinite = sNonFinite != 0;                   // uniform
             // slabs of consecutive groups of one segment are consecutive.  Uniform base (scalar
             // registers); the lanes add the 32-bit offset w_lane.
             const S* wchunk = Wq + (size_t)chunk_slot<FQ>(P.cpg, P.Cg, cc0) * per_slab;
@@ -248,6 +261,10 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
                     inside = inside && fabs(pa - pc) < (T)1;                // -1 < p < size, false for NaN
                     u[a] = (int)fl - tg_.hb[a];
                     inhalo = inhalo && (unsigned)u[a] < (unsigned)(H.hext[sa] - 1);
+                }
+                if (halo_nonfinite) {
+#pragma unroll
+                    for (int a = 0; a < ND; ++a) inhalo = inhalo && pq[a] > (T)0 && pq[a] < (T)(P.in[slot<ND>(a)] - 1);
                 }
                 const bool near = inside && inhalo, far = inside && !inhalo;
                 unsigned base;

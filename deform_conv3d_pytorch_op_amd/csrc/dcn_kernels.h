@@ -8,6 +8,7 @@
 // its channels (the reference recomputes them per channel).
 #pragma once
 #include "dcn_device.h"
+#include <limits>
 
 
 namespace dcn {
@@ -328,9 +329,21 @@ __device__ inline void halo_table(const Params& P, const HaloPlan& H, const Tile
 // Stage `nch` channels of the halo channel-interleaved, [halo voxel][CCH]: the CCH channel values of a voxel sit
 // next to each other, so one wide LDS read fetches a corner of all of them (missing channels of a
 // short last chunk and halo voxels outside the volume are stored as zero).
+//
+// Bank swizzle (float, CCH = 8).  A lane fetches four channels of a corner with one 16-byte read; with
+// 32 bytes per voxel the reads of one instruction -- the same four-channel group of 64 voxels -- would
+// only ever touch half of the LDS banks.  Voxel v therefore stores its four-channel group gq at
+// position gq ^ (v mod groups): the same group of neighbouring voxels lands in different banks, and a
+// read instruction spreads over all of them.  (Measured on 3-D layers, where the corner reads weigh
+// most: the 16-channel chunks of 2-D layers lose more to the selects of the staging loop and to the
+// padded halo rows than the reads gain.)
+template <typename T, int CCH>
+__host__ __device__ inline constexpr int swizzle_groups() { return (sizeof(T) == 4 && CCH == 8) ? CCH / 4 : 1; }
 template <typename T, int CCH, int WGS>
 __device__ inline void halo_stage_interleaved(const Params& P, const HaloPlan& H, const T* __restrict__ chan0, int nch,
-                                              const unsigned* __restrict__ sTab, T* __restrict__ sIn) {
+                                              const unsigned* __restrict__ sTab, T* __restrict__ sIn, int* __restrict__ nonfinite) {
+    constexpr int GPV = swizzle_groups<T, CCH>();
+    bool bad = false;                  // a NaN or an infinity among the staged values
     for (int v = threadIdx.x; v < H.hvol; v += WGS) {
         const unsigned t = sTab[v];
         const unsigned g = t == ~0u ? 0u : t;
@@ -339,8 +352,30 @@ __device__ inline void halo_stage_interleaved(const Params& P, const HaloPlan& H
         for (int c = 0; c < CCH; ++c) val[c] = chan0[(size_t)min(c, nch - 1) * P.inV + g];   // CCH loads in flight
         // cells outside the volume hold zero: samples in the rim read them with weight zero
 #pragma unroll
-        for (int c = 0; c < CCH; ++c) sIn[(size_t)v * CCH + c] = (c < nch && t != ~0u) ? val[c] : (T)0;
+        for (int c = 0; c < CCH; ++c) bad = bad || !(fabs(val[c]) <= std::numeric_limits<T>::max());
+#pragma unroll
+        for (int c = 0; c < CCH; ++c) val[c] = (c < nch && t != ~0u) ? val[c] : (T)0;
+        if constexpr (GPV > 1) {
+            const int sw = v & (GPV - 1);
+#pragma unroll
+            for (int gq = 0; gq < GPV; ++gq) {          // slot gq of the voxel holds group gq ^ sw
+                T o4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    T x = val[e];                        // sw == gq
+#pragma unroll
+                    for (int src = 0; src < GPV; ++src) x = (gq ^ sw) == src ? val[src * 4 + e] : x;
+                    o4[e] = x;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sIn[(size_t)v * CCH + gq * 4 + e] = o4[e];
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < CCH; ++c) sIn[(size_t)v * CCH + c] = val[c];
+        }
     }
+    if (bad) *nonfinite = 1;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -807,7 +842,8 @@ __global__ __launch_bounds__(512) void weight_bounds_kernel(const T* __restrict_
 // that (positions of the block x taps) of the largest possible one -- all that a cell can receive
 // -- still fit 31 bits; the host allows it only while that leaves enough bits below that term.
 // wmax[1] then holds the largest column norm of the weight (colnorm_max_kernel).
-template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false, int BS = 1>
+template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false, int BS = 1,
+          int HE1 = 0, int HE2 = 0>
 __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
                                                                   const T* __restrict__ in,
                                                                   const T* __restrict__ off,
@@ -838,20 +874,24 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     constexpr int CPL = PAIR ? CCH / 2 : CCH;           // cell planes
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int hs = HS ? HS : H.hstride;
+    // HE1, HE2 > 0 fix the two inner halo extents at compile time (the host then launches this
+    // instantiation only for plans with exactly these extents): the distances between the corners of a
+    // sample become immediate offsets of the LDS instructions instead of per-corner address arithmetic
+    const int he1 = HE1 ? HE1 : H.hext[1], he2 = HE2 ? HE2 : H.hext[2];
     Cell* sG = reinterpret_cast<Cell*>(smem_raw);                                       // [CPL][hstride]
     T* sIn = reinterpret_cast<T*>(sG + (size_t)CPL * hs);                               // [hstride][CCH] if COORD: channels of a voxel side by side
     unsigned* sTab = reinterpret_cast<unsigned*>(sIn + (COORD ? (size_t)CCH * hs : 0));   // [hvol]
     constexpr int WGS = NW * 64;                        // threads per workgroup
-    __shared__ float sRed[NW];
+    __shared__ float sRed[NW], sSum[NW], sAmax[NW];
+    __shared__ int sNonFinite;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     // Work items are (tile, deformable group) pairs.  The first `whole` workgroups of the launch take
     // one item each; every later item is shared by csplit workgroups, of which workgroup cz takes
     // every csplit-th channel chunk: finer work at the end of the launch fills the last, ragged
     // round of workgroups.  The grad_offset contributions of the channel chunks of a shared item meet
-    // through float atomics on a zero-filled buffer (the host passes goff_atomic = 1 when the launch
-    // has shared items and has cleared the buffer); the single owner of an item stores the first
-    // chunk's values and then the running sum.
+    // through float atomics on a zero-filled buffer; the single owner of an item stores the first
+    // chunk's values and then the running sum (or uses the atomics too: goff_atomic = 1).
     unsigned item;
     int cz = 0, cs = 1;
     if (blockIdx.x < whole) item = xcd_contiguous(blockIdx.x, whole);
@@ -864,8 +904,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     const unsigned nt = (unsigned)P.N * P.tiles;
     const int dg = item / nt;
     // an item that several workgroups share needs the atomics (the host has zero-filled grad_offset);
-    // the only owner of an item stores the running sum over its chunks instead
-    goff_atomic = cs > 1 ? 1 : 0;
+    // the only owner of an item stores the running sum over its chunks instead, unless the host asks for
+    // atomics there as well (goff_atomic: layers with so few grad_offset elements that the atomics cost
+    // less than the loads of the running sum)
+    goff_atomic = cs > 1 ? 1 : goff_atomic;
 
     TileGeo<ND> tg;
     tile_decode<ND>(P, H, item % nt, tg);
@@ -911,6 +953,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         const unsigned b_byte_last = (klast * KL + q < P.M ? b_off : pos) * (unsigned)sizeof(T);
         T b_reg[BREG ? NS * AB * BS : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share); PAIR: of the squares
+        float amax = 0.f;                           // PAIR: largest |grad_output| seen (squares of tiny values underflow)
         if constexpr (BREG) {
             // held unmasked (rows past M meet zero weight rows, columns outside the volume are never
             // used): a masked load becomes a conditional one, issued alone with a full wait behind it
@@ -928,7 +971,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
             for (int k = 0; k < NS * AB * BS; ++k) {
                 const float bk = (float)b_reg[k];
-                sabs += (valid && (k < kl || (k == kl && kl * KL + q < P.M))) ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
+                const bool counts = valid && (k < kl || (k == kl && kl * KL + q < P.M));
+                sabs += counts ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
+                if constexpr (PAIR) amax = counts ? fmaxf(amax, fabsf(bk)) : amax;
             }
         } else {
             // unconditional loads, eight in flight, masked when they are summed (a masked load
@@ -945,7 +990,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 for (int k = 0; k < AB; ++k) {
                     const int kk_ = k0 + k;
                     const float bk = (float)bv[k];
-                    sabs += (valid && (kk_ < klast || (kk_ == klast && klast * KL + q < P.M))) ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
+                    const bool counts = valid && (kk_ < klast || (kk_ == klast && klast * KL + q < P.M));
+                    sabs += counts ? (PAIR ? bk * bk : fabsf(bk)) : 0.f;
+                    if constexpr (PAIR) amax = counts ? fmaxf(amax, fabsf(bk)) : amax;
                 }
             }
         }
@@ -957,28 +1004,50 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         unsigned sbits = __float_as_uint(fabsf(sabs));
 #pragma unroll
         for (int sh = 1; sh < TN; sh <<= 1) sbits = max(sbits, (unsigned)__shfl_xor((int)sbits, sh));
+        // paired cells: also the sum over the block's positions of the norm of grad_output over the
+        // output channels (every lane of a position holds its full sum of squares by now)
+        float nsum = PAIR ? sqrtf(sabs) : 0.f;
+        if constexpr (PAIR) {
+#pragma unroll
+            for (int sh = 1; sh < TN; sh <<= 1) nsum += __shfl_xor(nsum, sh);
+#pragma unroll
+            for (int sh = 1; sh < 64; sh <<= 1) amax = fmaxf(amax, __shfl_xor(amax, sh));
+        }
         __syncthreads();
-        if (lane == 0) sRed[wave] = __uint_as_float(sbits);
+        if (lane == 0) { sRed[wave] = __uint_as_float(sbits); sSum[wave] = nsum; sAmax[wave] = amax; }
         __syncthreads();
         unsigned smaxb = 0u;
+        float ssum = 0.f, gmax = 0.f;
 #pragma unroll
-        for (int w8 = 0; w8 < NW; ++w8) smaxb = max(smaxb, __float_as_uint(sRed[w8]));
+        for (int w8 = 0; w8 < NW; ++w8) { smaxb = max(smaxb, __float_as_uint(sRed[w8])); ssum += sSum[w8]; gmax = fmaxf(gmax, sAmax[w8]); }
         int ex = 0;
         // paired cells: |term| <= largest column norm of W x largest norm of grad_output over the
         // output channels (0.1 % slack for the rounding of those two and of the MFMA sums)
         const float bound = PAIR ? 1.001f * wmax[1] * sqrtf(__uint_as_float(smaxb)) : 8.f * wmax[0] * __uint_as_float(smaxb);
+        // paired cells: all that one cell can receive.  A (tap, position) spreads at most |grad column| over
+        // its corners (their weights add up to one), so a cell's terms add up to at most the sum over the
+        // block's positions and the taps of that bound -- far less than (number of terms) x (largest term)
+        // when a few positions carry most of grad_output
+        const float bound_cell = PAIR ? 1.001f * wmax[1] * (float)P.kV * ssum : 0.f;
         // the LDS cells need a finite bound; without one this workgroup scatters through the far path
         // (float cells need the exponent; and with either cell type a corner that carries weight zero
         // would receive 0 * inf = NaN where the reference adds nothing)
-        const bool cells_ok = bound < 3.0e38f;                        // false for NaN
+        // (and a block whose grad_output is so small that its squares underflow: the bound is then not
+        // trustworthy, and the workgroup takes the far path too rather than rounding its gradient away)
+        const bool cells_ok = bound < 3.0e38f && bound_cell < 3.0e38f && !(PAIR && gmax > 0.f && gmax < 1e-18f);            // false for NaN
         if (bound > 0.f && bound < 3.0e38f) (void)frexpf(bound, &ex);
         double scale = ldexp(1.0, 30 - ex), inv_scale = ldexp(1.0, ex - 30);
         float scale32 = 1.f;
         if constexpr (PAIR) {
-            // all the terms a cell can receive, each at the bound, stay below 2^31; and a single term
-            // below 2^22 (the float conversion of add2)
-            const double terms = (double)(NW * TN) * P.kV;
-            scale = bound > 0.f && bound < 3.0e38f ? 0.99 * (terms > 512.0 ? 2147483648.0 / terms : 4194304.0) / (double)bound : 1.0;
+            // a single term stays below 2^22 (the float conversion of add2) and all the terms a cell can
+            // receive together below 2^31 (their roundings, half a unit each for at most NW * TN * kV
+            // terms, fit the one per cent of slack)
+            if (bound > 0.f && cells_ok) {
+                const double s_term = 4194304.0 / (double)bound;
+                const double s_cell = bound_cell > 0.f ? 2147483648.0 / (double)bound_cell : s_term;
+                scale = 0.99 * (s_term < s_cell ? s_term : s_cell);
+            } else
+                scale = 1.0;
             scale32 = (float)(scale < 1e30 ? scale : 1e30);       // (a denormal bound: keep the scale a finite float)
             scale = (double)scale32;                 // the flush divides by exactly what the terms were multiplied with
             inv_scale = 1.0 / scale;
@@ -987,11 +1056,18 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         for (int cc0 = rb; cc0 < re; cc0 += CCH) {
             if ((chunk_no++) % cs != cz) continue;          // another workgroup's chunk (uniform)
             const int nch = min(CCH, re - cc0);
+            if (threadIdx.x == 0) sNonFinite = 0;
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < (PAIR ? (nch + 1) / 2 : nch); ++c)
                 for (int v = threadIdx.x; v < H.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
-            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, H, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn);
+            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, H, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn, &sNonFinite);
             __syncthreads();
+            // Non-finite input values in this halo: the branch-free sampler reads the cell next to a
+            // collapsed corner with weight 0, and 0 * inf would be NaN where the reference never
+            // touches that voxel (deform3d/lib/deform_conv3d_cuda_kernel.cu:24-26).  Samples in the
+            // collapse zones (p <= 0 or p >= size - 1 on some axis) then take the far path, which
+            // follows the reference's corner rule.
+            const bool halo_nonfinite = COORD && sNonFinite != 0;          // uniform
 
             // Grad-column tile of a pass: row i = (tap tap0 + i / CCH, channel cc0 + i % CCH); taps past
             // the last one read zero padding (or rows that are ignored below).  The MFMAs of pass p+1
@@ -1021,9 +1097,13 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             };
             // steps [k_begin, ksteps) of one pass in a software-pipelined loop of their own: the whole
             // first pass, and what the tap slots cannot take when M is large
+            // (two operand sets that swap roles from batch to batch, two batches per loop trip: copying
+            // "next" into "current" costs 2 * AB register moves per batch whenever the register
+            // allocator cannot merge the sets, on the same issue port as the MFMAs)
             auto gemm_tail = [&](typename MM::Acc& dd, const T* wp, int k_begin) {
-                T a_nx[AB], b_nx[AB];
-                load_batch(a_nx, b_nx, wp, k_begin);
+                T a_s[2][AB], b_s[2][AB];
+                load_batch(a_s[0], b_s[0], wp, k_begin);
+                int k0 = k_begin;
                 if (PACKW && ksteps - k_begin >= 96) {
                     // Long reductions (M >= 192 float): the next batch is requested in the same block
                     // as this batch's MFMAs (past the last step the padded slab's last batch is read
@@ -1031,13 +1111,23 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     // between the MFMAs.  The wavefronts of a workgroup run in step, so a separate load
                     // phase leaves the matrix pipe idle in all of them at once.  (Short reductions lose
                     // more to the one redundant batch than they gain.)
-                    for (int k0 = k_begin; k0 < ksteps; k0 += AB) {
-                        T a_cu[AB], b_cu[AB];
+                    const int k_last = (int)(wpass / 64) - AB;
+                    // Batches all of whose steps are real ones for every lane need no clamping of the
+                    // grad_output rows: two scalar adds per load instead of a dozen scalar instructions,
+                    // which a wavefront has to issue between two MFMAs.
+                    const int kfast_end = P.M % KL == 0 ? klast + 1 : klast;      // steps [0, kfast_end) load without a clamp
+                    auto load_fast = [&](T* a_nx, T* b_nx, int k0f) {
+                        asm volatile("" : "+s"(k0f));
+                        const T* wb = wp + (size_t)k0f * wstep;
+                        const char* gk = reinterpret_cast<const char*>(gbase + (size_t)k0f * gstep);
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) { a_cu[k] = a_nx[k]; b_cu[k] = b_nx[k]; }
-                        load_batch(a_nx, b_nx, wp, min(k0 + AB, (int)(wpass / 64) - AB));
-#pragma unroll
-                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_cu[k], b_cu[k], dd);
+                        for (int k = 0; k < AB; ++k) {
+                            a_nx[k] = (wb + (unsigned)k * (unsigned)wstep)[a_off];
+                            b_nx[k] = *reinterpret_cast<const T*>(gk + b_byte);
+                            gk += gstep * sizeof(T);
+                        }
+                    };
+                    auto deal = [&]() {
 #pragma unroll
                         for (int k = 0; k < AB; ++k) {
                             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
@@ -1045,18 +1135,50 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                             __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);      // vector
                             __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);      // two loads
                         }
+                    };
+                    if constexpr (!BREG) {
+                        for (; k0 + 3 * AB <= kfast_end; k0 += 2 * AB) {
+                            load_fast(a_s[1], b_s[1], k0 + AB);
+#pragma unroll
+                            for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                            deal();
+                            load_fast(a_s[0], b_s[0], k0 + 2 * AB);
+#pragma unroll
+                            for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[1][k], b_s[1][k], dd);
+                            deal();
+                        }
+                    }
+                    for (; k0 + AB < ksteps; k0 += 2 * AB) {
+                        load_batch(a_s[1], b_s[1], wp, min(k0 + AB, k_last));
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                        deal();
+                        load_batch(a_s[0], b_s[0], wp, min(k0 + 2 * AB, k_last));
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[1][k], b_s[1][k], dd);
+                        deal();
+                    }
+                    if (k0 < ksteps) {
+#pragma unroll
+                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
                     }
                     return;
                 }
-                for (int k0 = k_begin; k0 < ksteps; k0 += AB) {
-                    T a_cu[AB], b_cu[AB];
-#pragma unroll
-                    for (int k = 0; k < AB; ++k) { a_cu[k] = a_nx[k]; b_cu[k] = b_nx[k]; }
-                    if (k0 + AB < ksteps) load_batch(a_nx, b_nx, wp, k0 + AB);
+                for (; k0 + AB < ksteps; k0 += 2 * AB) {
+                    load_batch(a_s[1], b_s[1], wp, k0 + AB);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_cu[k], b_cu[k], dd);
+                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
                     __builtin_amdgcn_sched_barrier(0);
+                    if (k0 + 2 * AB < ksteps) load_batch(a_s[0], b_s[0], wp, k0 + 2 * AB);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[1][k], b_s[1][k], dd);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (k0 < ksteps) {
+#pragma unroll
+                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
                 }
             };
             // register-resident operand: the batches of a pass past those that ride on the tap slots
@@ -1098,8 +1220,11 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             // plain loads and stores that stay in the L2 between two chunks, where float atomics are
             // limited to about one per clock and L2 channel (130 M of them per call on a 64-channel
             // 3x3x3 layer of 200 k positions)
+            // (3-D kernels only: the short tap slots of the 2-D kernels lose more to the extra loads than
+            // their few grad_offset elements cost in atomics, so the host asks for atomics there)
+            constexpr bool RMW = COORD && ND == 3;
             T p_buf[2][ND];
-            const bool rmw_prev = COORD && !goff_atomic && !first_chunk;        // uniform
+            const bool rmw_prev = RMW && !goff_atomic && !first_chunk;        // uniform
             static_assert(NS % 2 == 0, "offset buffers alternate within a pass");
             // Kernel coordinates of this lane's tap in the next slot, counted up with the slots (the
             // taps of consecutive slots are TP / NS apart for every lane).  They live in registers: a
@@ -1121,7 +1246,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 const T* ob = off_dg + (size_t)tu * ND * P.outV;
 #pragma unroll
                 for (int a = 0; a < ND; ++a) o_nx[a] = (ob + (size_t)a * P.outV)[lo];
-                if constexpr (COORD) {
+                if constexpr (RMW) {
                     if (rmw_prev) {
                         const T* gb = goff_dg + (size_t)tu * ND * P.outV;
 #pragma unroll
@@ -1157,7 +1282,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                     for (int a = 0; a < ND; ++a) {
                         if (goff_atomic) { if (pend_ga[a] != (T)0) atomic_add(gp + (size_t)a * P.outV, pend_ga[a]); }
-                        else gp[(size_t)a * P.outV] = pend_ga[a];       // (the earlier chunks' sum is part of it)
+                        else if (RMW || first_chunk) gp[(size_t)a * P.outV] = pend_ga[a];       // (3-D: the earlier chunks' sum is part of it)
+                        else gp[(size_t)a * P.outV] += pend_ga[a];
                     }
                 }
                 pend = false;
@@ -1167,8 +1293,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             unsigned coff[NC];
 #pragma unroll
             for (int i = 0; i < NC; ++i)
-                coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * H.hext[1] + ((i >> 1) & 1)) * H.hext[2] + (i & 1))
-                                  : (unsigned)(((i >> 1) & 1) * H.hext[2] + (i & 1));
+                coff[i] = ND == 3 ? (unsigned)((((i >> 2) & 1) * he1 + ((i >> 1) & 1)) * he2 + (i & 1))
+                                  : (unsigned)(((i >> 1) & 1) * he2 + (i & 1));
 
             for (int tap0 = 0; tap0 < P.kV; tap0 += TP) {
                 const typename MM::Acc d = d_next;
@@ -1225,10 +1351,16 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         u[a] = (int)fl - tg.hb[a];
                         inhalo = inhalo && (unsigned)u[a] < (unsigned)(H.hext[s] - 1);
                     }
+                    {   // (mask arithmetic, no branch)
+                        bool all_intr = true;
+#pragma unroll
+                        for (int a = 0; a < ND; ++a) all_intr = all_intr & intr[a];
+                        inhalo = inhalo & (all_intr | !halo_nonfinite);
+                    }
                     const bool near = inside && inhalo, far = inside && !inhalo;
                     unsigned base;
-                    if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], H.hext[1]) + u[1], H.hext[2]) + u[2]);
-                    else base = (unsigned)(__mul24(u[0], H.hext[2]) + u[1]);
+                    if constexpr (ND == 3) base = (unsigned)(__mul24(__mul24(u[0], he1) + u[1], he2) + u[2]);
+                    else base = (unsigned)(__mul24(u[0], he2) + u[1]);
                     base = near ? base : 0u;       // lanes without a sample in the halo read cell 0 and add nothing
                     T cw[NC];
                     if constexpr (ND == 3) {       // multiplied in the reference's order (w_l * w_h * w_w)
@@ -1264,10 +1396,26 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         T vv[NC][RW];
                         if constexpr (COORD) {
                             const T* ip = sIn + (size_t)base * CCH;
+                            constexpr int GPV = swizzle_groups<T, CCH>();
+                            if constexpr (GPV > 1) {
+                                // the four-channel group of this round sits at slot (group ^ voxel mod GPV) of its
+                                // voxel (halo_stage_interleaved); the innermost halo extent is a multiple of GPV
+                                // (host), so a corner's voxel is base + (i & 1) modulo GPV
+                                static_assert(RW == 4, "a round reads one four-channel group");
+                                const int grp = row_ch(ts * RPS + h * RW, q) / 4;
+                                const T* ipx[2];
+                                ipx[0] = ip + (((unsigned)grp ^ (base & (GPV - 1))) << 2);
+                                ipx[1] = ip + (((unsigned)grp ^ ((base + 1) & (GPV - 1))) << 2);
 #pragma unroll
-                            for (int i = 0; i < NC; ++i)
+                                for (int i = 0; i < NC; ++i)
 #pragma unroll
-                                for (int rr = 0; rr < RW; ++rr) vv[i][rr] = ip[coff[i] * CCH + row_ch(ts * RPS + h * RW + rr, q)];
+                                    for (int rr = 0; rr < RW; ++rr) vv[i][rr] = ipx[i & 1][coff[i] * CCH + rr];
+                            } else {
+#pragma unroll
+                                for (int i = 0; i < NC; ++i)
+#pragma unroll
+                                    for (int rr = 0; rr < RW; ++rr) vv[i][rr] = ip[coff[i] * CCH + row_ch(ts * RPS + h * RW + rr, q)];
+                            }
                         }
                         // the next pass's MFMAs of this slot, in uniform control flow
                         if (do_mma) {
@@ -1410,7 +1558,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         pend = slot_ok && owner;
                         pend_tap = tap;
 #pragma unroll
-                        for (int a = 0; a < ND; ++a) pend_ga[a] = rmw_prev ? ga[a] + p_buf[ts & 1][a] : ga[a];
+                        for (int a = 0; a < ND; ++a) {
+                            if constexpr (RMW) pend_ga[a] = rmw_prev ? ga[a] + p_buf[ts & 1][a] : ga[a];
+                            else pend_ga[a] = ga[a];
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);      // one tap slot at a time: keeps the live register set small
                 }

@@ -84,6 +84,6 @@ def test_small_cases_under_knob(extra):
     env = dict(os.environ)
     env.update(extra)
     r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.join(ROOT, "tests", "test_gpu_parity.py"), "-q", "-x",
-                        "-m", "gpu", "-k", "small_cases or golden or non_finite or oob_offset_grad or random_geometries or random_medium", "--timeout", "120", "--timeout-method", "thread"],
+                        "-m", "gpu", "-k", "small_cases or golden or non_finite or heavy_tailed or oob_offset_grad or random_geometries or random_medium", "--timeout", "120", "--timeout-method", "thread"],
                        cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-3000:]
