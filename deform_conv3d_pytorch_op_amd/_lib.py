@@ -15,6 +15,7 @@ _c_int, _c_vp, _c_sz = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 _lib = None
 
 N_GEOM = {3: 23, 2: 17}     # number of int arguments of DCN3D_GEOMETRY / DCN2D_GEOMETRY
+N_CONV2D_GEOM = 16          # ... of CONV2D_GEOMETRY
 
 
 class DcnError(RuntimeError):
@@ -51,6 +52,16 @@ def load():
             if nd == 3 and suf in ("f32", "f64"):
                 f = getattr(L, "dcn3d_backward_input_offset_flags_%s" % suf)
                 f.restype, f.argtypes = _c_int, [_c_vp] * 6 + geom + tail + [ctypes.c_uint]
+    L.conv2d_workspace_bytes.restype = _c_sz
+    L.conv2d_workspace_bytes.argtypes = [_c_int] * 4 + [_c_sz, _c_sz, _c_int, _c_int]
+    cgeom = [_c_int] * N_CONV2D_GEOM
+    for suf in ("f32", "f64"):
+        f = getattr(L, "conv2d_forward_" + suf)
+        f.restype, f.argtypes = _c_int, [_c_vp] * 4 + cgeom + tail
+        f = getattr(L, "conv2d_backward_input_" + suf)
+        f.restype, f.argtypes = _c_int, [_c_vp] * 3 + cgeom + tail
+        f = getattr(L, "conv2d_backward_weight_" + suf)
+        f.restype, f.argtypes = _c_int, [_c_vp] * 3 + cgeom + tail
     L.dcn3d_forward_noalloc_f32.restype = _c_int
     L.dcn3d_forward_noalloc_f32.argtypes = [_c_vp] * 5 + [_c_int] * N_GEOM[3] + [_c_vp]
     if L.dcn_version() != 1:
@@ -69,6 +80,7 @@ EXPORTS = ["dcn_version", "dcn_arch", "dcn_last_error", "dcn_workspace_bytes", "
     for nd in (2, 3) for op in ("forward", "backward_input_offset", "backward_weight")
     for suf in ("f32", "f64", "bf16", "f16")] + [
     "dcn3d_backward_input_offset_flags_f32", "dcn3d_backward_input_offset_flags_f64",
-    "dcn3d_forward_noalloc_f32"]
+    "dcn3d_forward_noalloc_f32", "conv2d_workspace_bytes"] + [
+    "conv2d_%s_%s" % (op, suf) for op in ("forward", "backward_input", "backward_weight") for suf in ("f32", "f64")]
 NOALLOC_SCRATCH_BYTES = 8 << 20
 FLAG_OOB_OFFSET_GRAD_ZERO = 1

@@ -703,15 +703,19 @@ int weight_bounds(const Params& P, const T* w, float* out, hipStream_t s) {
     return check_launch("weight_bounds_kernel");
 }
 
+constexpr unsigned FLAG_INPUT_ONLY = 0x100u;     // internal: see backward_input_offset
 template <typename T, int ND>
 int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* off, const T* gout, T* gin,
                           T* goff, void* ws, size_t ws_bytes, hipStream_t s, unsigned flags = 0) {
     Params P;
     if (int rc = validate(g, P)) return rc;
-    if (flags & ~(unsigned)DCN_FLAG_OOB_OFFSET_GRAD_ZERO) return fail(DCN_E_ARGUMENT, "unknown flag");
+    if (flags & ~(unsigned)(DCN_FLAG_OOB_OFFSET_GRAD_ZERO | FLAG_INPUT_ONLY)) return fail(DCN_E_ARGUMENT, "unknown flag");
     if (int rc = device_info(nullptr)) return rc;
     P.oob_zero = (flags & DCN_FLAG_OOB_OFFSET_GRAD_ZERO) ? 1 : 0;
-    if (!in || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
+    // grad_input alone (the plain convolution's backward-to-input, which is not given the input): the
+    // scatter kernels need no input values; `goff` is then scratch for the one kernel that writes it anyway
+    const bool input_only = (flags & FLAG_INPUT_ONLY) != 0;
+    if ((!in && !input_only) || !w || !off || !gout || !gin || !goff) return fail(DCN_E_ARGUMENT, "null tensor pointer");
     bwd_data_weight_pad<T>(P.M, P.Cg, P.Mp, P.Cgp);
     const size_t wbytes = bwd_data_weight_bytes<T>(P.M, P.Cg, P.kV, P.G, P.cpg);
     const size_t tbytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
@@ -877,7 +881,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     FusedPlan fp[MAX_PLANS];
     int margins[MAX_PLANS];
     const int nmargins = plan_margins(ND, margins);
-    if (scatter_in_lds() && fused_coord() && plan_fused(margins[0], fp[0])) {
+    if (scatter_in_lds() && fused_coord() && !input_only && plan_fused(margins[0], fp[0])) {
         // Wider halos for offsets that reach further; the choice is made on the device, see
         // PlanChoice.  A plan whose weights want another lane order gets a packed copy of its own in
         // the region of the channels-last input, which this path does not use.
@@ -990,8 +994,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         hipLaunchKernelGGL(fill_zero_kernel<T>, dim3((unsigned)((pad + 255) / 256)), dim3(256), 0, s, wt + used, pad);
         if (int rc = check_launch("fill_zero_kernel")) return rc;
     }
-    hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
-    if (int rc = check_launch("to_channels_last_kernel")) return rc;
+    if (!input_only) {
+        hipLaunchKernelGGL(to_channels_last_kernel<T>, tgrid, tblock, 0, s, in, in_cl, P.C_in, P.inV);
+        if (int rc = check_launch("to_channels_last_kernel")) return rc;
+    }
     Params Ph = P;
     bool halo = scatter_in_lds() && plan_halo<T, ND>(Ph, scatter_budget(), default_margin(), 8, 8);
     if (halo && (long long)Ph.N * Ph.tiles * Ph.DG > 0x7fffffffLL) halo = false;
@@ -1007,13 +1013,15 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     const dim3 grid((unsigned)P.N * P.tiles, (unsigned)P.DG);
     if (halo) {
         T* none = nullptr;
+        if (!input_only)
         switch (mk) {      // register-resident grad_output slab when M is small enough
             case 8: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 8>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             case 16: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 16>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             case 32: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 32>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
             default: hipLaunchKernelGGL((backward_data_kernel<T, ND, false, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, none, goff); break;
         }
-        if (int rc = check_launch("backward_data_kernel")) return rc;
+        if (!input_only)
+            if (int rc = check_launch("backward_data_kernel")) return rc;
         const size_t lds = (size_t)Ph.cchunk * Ph.hstride * 8 + (size_t)Ph.hvol * 4;
         if (int rc = absmax<T>(w, (size_t)P.C_out * P.Cg * P.kV, wmax, s)) return rc;
         const dim3 hgrid((unsigned)Ph.N * Ph.tiles * Ph.DG);
@@ -1035,6 +1043,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     const unsigned fblocks = (unsigned)((nelem + 1023) / 1024 > 8192 ? 8192 : (nelem + 1023) / 1024);
     hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fblocks), dim3(256), 0, s, gin_cl, nelem);
     if (int rc = check_launch("fill_zero_kernel")) return rc;
+    if (input_only) {       // the kernel reads input values for the grad_offset it also writes (into scratch here)
+        hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(fblocks), dim3(256), 0, s, in_cl, nelem);
+        if (int rc = check_launch("fill_zero_kernel")) return rc;
+    }
     hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 0>), grid, dim3(WG), 0, s, P, in_cl, off, wt, gout, gin_cl, goff);
     if (int rc = check_launch("backward_data_kernel")) return rc;
     hipLaunchKernelGGL(add_from_channels_last_kernel<T>, tgrid, tblock, 0, s, gin_cl, gin, P.C_in, P.inV);
@@ -1254,6 +1266,50 @@ int backward_weight16(const Geometry& g, const S* in, const S* off, const S* gou
     return narrow(fgw, gw, z.w, s);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Plain 2-D convolution: the reference's conv2d package (conv2d/lib/conv2d_cuda.cpp:77-290, kernels
+// conv2d/lib/conv2d_cuda_kernel.cu:25-169: im2col / col2im with integer taps and one GEMM per sample
+// and group).  It is the 2-D deformable layer with every offset zero, one deformable group and the
+// dilation-aware output size (conv2d/lib/conv2d_cuda.cpp:20-22), so it runs on the same kernels: a
+// zero offset tensor at the front of the workspace, behind it scratch for the grad_offset that
+// one fallback kernel of backward-to-input writes, then the deformable layer's own workspace.
+template <typename T> size_t conv2d_zero_bytes(int N, int kV, size_t outV) { return align256((size_t)N * 2 * kV * outV * sizeof(T)); }
+template <typename T>
+int conv2d_offsets(const Geometry& g, void* ws, size_t ws_bytes, hipStream_t s, T** off, T** scratch, void** rest, size_t* rest_bytes) {
+    if (g.N <= 0 || g.out[1] <= 0 || g.out[2] <= 0 || g.k[1] <= 0 || g.k[2] <= 0) return fail(DCN_E_ARGUMENT, "batch / output / kernel extents must be positive");
+    const size_t zb = conv2d_zero_bytes<T>(g.N, g.k[1] * g.k[2], (size_t)g.out[1] * g.out[2]);
+    if (!ws || ws_bytes < 2 * zb) return fail(DCN_E_WORKSPACE, "workspace too small");
+    *off = static_cast<T*>(ws);
+    *scratch = reinterpret_cast<T*>(static_cast<char*>(ws) + zb);
+    *rest = static_cast<char*>(ws) + 2 * zb;
+    *rest_bytes = ws_bytes - 2 * zb;
+    const size_t n = zb / sizeof(T);
+    const unsigned blocks = (unsigned)((n + 1023) / 1024 > 4096 ? 4096 : (n + 1023) / 1024);
+    hipLaunchKernelGGL(fill_zero_kernel<T>, dim3(blocks), dim3(256), 0, s, *off, n);
+    return check_launch("fill_zero_kernel");
+}
+template <typename T>
+int conv2d_forward(Geometry g, const T* in, const T* w, const T* bias, T* out, void* ws, size_t ws_bytes, hipStream_t s) {
+    g.cpg = g.C_in;
+    T *off, *scratch; void* rest; size_t rest_bytes;
+    if (int rc = conv2d_offsets<T>(g, ws, ws_bytes, s, &off, &scratch, &rest, &rest_bytes)) return rc;
+    return forward<T, 2>(g, in, w, off, bias, out, rest, rest_bytes, s);
+}
+template <typename T>
+int conv2d_backward_input(Geometry g, const T* w, const T* gout, T* gin, void* ws, size_t ws_bytes, hipStream_t s) {
+    g.cpg = g.C_in;
+    T *off, *scratch; void* rest; size_t rest_bytes;
+    if (int rc = conv2d_offsets<T>(g, ws, ws_bytes, s, &off, &scratch, &rest, &rest_bytes)) return rc;
+    return backward_input_offset<T, 2>(g, nullptr, w, off, gout, gin, scratch, rest, rest_bytes, s, FLAG_INPUT_ONLY);
+}
+template <typename T>
+int conv2d_backward_weight(Geometry g, const T* in, const T* gout, T* gw, void* ws, size_t ws_bytes, hipStream_t s) {
+    g.cpg = g.C_in;
+    T *off, *scratch; void* rest; size_t rest_bytes;
+    if (int rc = conv2d_offsets<T>(g, ws, ws_bytes, s, &off, &scratch, &rest, &rest_bytes)) return rc;
+    return backward_weight<T, 2>(g, in, off, gout, gw, rest, rest_bytes, s);
+}
+
 Geometry geo3(int batch, int input_c, int output_c, int input_l, int input_h, int input_w, int output_l,
               int output_h, int output_w, int kernel_l, int kernel_h, int kernel_w, int pad_l, int pad_h,
               int pad_w, int stride_l, int stride_h, int stride_w, int dilation_l, int dilation_h,
@@ -1377,6 +1433,7 @@ int dcn3d_forward_noalloc_f32(const float* input, const float* weight, const flo
                                                 const T* grad_output, T* grad_input, T* grad_offset,                \
                                                 DCN3D_GEOMETRY, void* workspace, size_t workspace_bytes,            \
                                                 void* stream, unsigned flags) {                                     \
+        if (flags & ~(unsigned)DCN_FLAG_OOB_OFFSET_GRAD_ZERO) return fail(DCN_E_ARGUMENT, "unknown flag");          \
         return backward_input_offset<T, 3>(geo3(G3_ARGS), input, weight, offset, grad_output, grad_input,           \
                                            grad_offset, workspace, workspace_bytes,                                 \
                                            static_cast<hipStream_t>(stream), flags);                                \
@@ -1406,6 +1463,36 @@ int dcn3d_forward_noalloc_f32(const float* input, const float* weight, const flo
 
 DEFINE_OPS(f32, float)
 DEFINE_OPS(f64, double)
+
+size_t conv2d_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume, size_t output_volume,
+                              int kernel_volume, int group) {
+    const size_t inner = dcn_workspace_bytes_for(elem_size, batch, input_c, output_c, input_volume, output_volume, kernel_volume,
+                                                 group, input_c);
+    if (!inner || elem_size == 2) return 0;
+    const size_t zb = elem_size == 8 ? conv2d_zero_bytes<double>(batch, kernel_volume, output_volume)
+                                     : conv2d_zero_bytes<float>(batch, kernel_volume, output_volume);
+    return inner + 2 * zb;
+}
+#define C2_ARGS batch, input_c, output_c, input_h, input_w, output_h, output_w, kernel_h, kernel_w, pad_h, pad_w, \
+                stride_h, stride_w, dilation_h, dilation_w, input_c, group
+#define DEFINE_CONV2D(SUF, T)                                                                                       \
+    int conv2d_forward_##SUF(const T* input, const T* weight, const T* bias, T* output, CONV2D_GEOMETRY,            \
+                             void* workspace, size_t workspace_bytes, void* stream) {                               \
+        return conv2d_forward<T>(geo2(C2_ARGS), input, weight, bias, output, workspace, workspace_bytes,            \
+                                 static_cast<hipStream_t>(stream));                                                 \
+    }                                                                                                               \
+    int conv2d_backward_input_##SUF(const T* weight, const T* grad_output, T* grad_input, CONV2D_GEOMETRY,          \
+                                    void* workspace, size_t workspace_bytes, void* stream) {                        \
+        return conv2d_backward_input<T>(geo2(C2_ARGS), weight, grad_output, grad_input, workspace, workspace_bytes, \
+                                        static_cast<hipStream_t>(stream));                                          \
+    }                                                                                                               \
+    int conv2d_backward_weight_##SUF(const T* input, const T* grad_output, T* grad_weight, CONV2D_GEOMETRY,         \
+                                     void* workspace, size_t workspace_bytes, void* stream) {                       \
+        return conv2d_backward_weight<T>(geo2(C2_ARGS), input, grad_output, grad_weight, workspace,                 \
+                                         workspace_bytes, static_cast<hipStream_t>(stream));                        \
+    }
+DEFINE_CONV2D(f32, float)
+DEFINE_CONV2D(f64, double)
 
 #define DEFINE_OPS16(SUF, S)                                                                                        \
     int dcn3d_forward_##SUF(const void* input, const void* weight, const void* offset, const void* bias, void* output, \

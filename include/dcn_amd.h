@@ -169,6 +169,36 @@ int dcn2d_backward_weight_f64(const double *input, const double *offset, const d
                               double *grad_weight, DCN2D_GEOMETRY, void *workspace,
                               size_t workspace_bytes, void *stream);
 
+/* ---- plain 2-D convolution -------------------------------------------------------------------
+ * replaces the three symbols of the reference's conv2d package, conv2d/lib/conv2d_cuda.h:17-39
+ * (conv_forward_cuda, conv_backward_input_cuda, conv_backward_weight_cuda; host loops
+ * conv2d/lib/conv2d_cuda.cpp:77-290).  The reference's `columns` argument does not exist here.  The
+ * output extents follow the dilation-aware formula of conv2d/lib/conv2d_cuda.cpp:20-22,
+ * (input + 2 pad - dilation (kernel - 1) - 1) / stride + 1.  `bias` ([output_c] or NULL) is added in
+ * the epilogue (the reference adds it from Python, conv2d/conv2d_functions/conv2d_function.py:34-35);
+ * grad_input and grad_weight are accumulated into (the caller zero-fills them, as the reference's
+ * Function does).  backward_input is not given the input, like the reference's.  The layer runs as the
+ * 2-D deformable layer with every offset zero; the workspace (conv2d_workspace_bytes) holds that zero
+ * offset tensor in front of the deformable layer's own workspace. */
+#define CONV2D_GEOMETRY                                                                          \
+    int batch, int input_c, int output_c, int input_h, int input_w, int output_h, int output_w,  \
+    int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,                \
+    int dilation_h, int dilation_w, int group
+size_t conv2d_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
+                              size_t output_volume, int kernel_volume, int group);
+int conv2d_forward_f32(const float *input, const float *weight, const float *bias, float *output, CONV2D_GEOMETRY,
+                       void *workspace, size_t workspace_bytes, void *stream);
+int conv2d_forward_f64(const double *input, const double *weight, const double *bias, double *output, CONV2D_GEOMETRY,
+                       void *workspace, size_t workspace_bytes, void *stream);
+int conv2d_backward_input_f32(const float *weight, const float *grad_output, float *grad_input, CONV2D_GEOMETRY,
+                              void *workspace, size_t workspace_bytes, void *stream);
+int conv2d_backward_input_f64(const double *weight, const double *grad_output, double *grad_input, CONV2D_GEOMETRY,
+                              void *workspace, size_t workspace_bytes, void *stream);
+int conv2d_backward_weight_f32(const float *input, const float *grad_output, float *grad_weight, CONV2D_GEOMETRY,
+                               void *workspace, size_t workspace_bytes, void *stream);
+int conv2d_backward_weight_f64(const double *input, const double *grad_output, double *grad_weight, CONV2D_GEOMETRY,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- 16-bit storage, float32 accumulation ----------------------------------------------------
  * No counterpart in the reference, which instantiates float only
  * (deform3d/lib/deform_conv3d_cuda_kernel.cu:162-172).  Every tensor (input, weight, offset, bias,

@@ -19,7 +19,7 @@ def test_library_exports_every_declared_symbol():
     from deform_conv3d_pytorch_op_amd import _lib
     L = _lib.load()
     header = open(os.path.join(ROOT, "include", "dcn_amd.h")).read()
-    declared = set(re.findall(r"\b(dcn(?:2d|3d)?_[a-z0-9_]+)\s*\(", header))
+    declared = set(re.findall(r"\b((?:dcn(?:2d|3d)?|conv2d)_[a-z0-9_]+)\s*\(", header))
     assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(L, name), name
