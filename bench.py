@@ -1,6 +1,6 @@
 """Benchmark of the deformable-convolution hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5|all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5|all] [--no-cpu] [--dtype f32|f64]
 
 A step is one forward + backward (grad input, grad offset, grad weight) of one layer through the
 package's autograd Function on synthetic inputs already resident in HBM.  The default workload is
@@ -101,6 +101,8 @@ def run_config(name, a):
     from deform_conv3d_pytorch_op_amd.synthetic import make_case
 
     spec = CONFIGS[name]
+    if a.dtype is not None:             # the configuration's shapes in the other precision
+        spec = spec[:-1] + ({"f32": "float32", "f64": "float64"}[a.dtype],)
     dtype = getattr(torch, spec[-1])
     kw = dict(dtype=dtype, seed=0, bias=False)
     if a.offset_scale is not None:      # not the configuration's own offsets: U[-s, s]
@@ -198,7 +200,7 @@ def run_config(name, a):
     achieved = F / (kernel_ms[dominant] * 1e-3) / 1e12
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": round(achieved, 3), "peak": peak,
                 "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                "traffic": measured_traffic(name, dominant) if a.offset_scale is None else None,
+                "traffic": measured_traffic(name, dominant) if a.offset_scale is None and a.dtype is None else None,
                 "ms": round(kernel_ms[dominant], 4),
                 "algorithmic_flops": F, "algorithmic_bytes": ab[dominant],
                 "hbm_frac_at_algorithmic_bytes": round(ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
@@ -223,14 +225,25 @@ def run_config(name, a):
             orc.forward(xs, offs, c["w"], None, *cfg, acc64=False)
             orc.backward(xs, offs, c["w"], gs, None, *cfg, acc64=False)
             return time.perf_counter() - t0
-        first = once()                         # also warms the thread pool; not counted
-        reps = max(3, min(25, int(12.0 / max(first, 1e-3))))      # about 12 s of host work per configuration
-        times = [once() for _ in range(reps)]
-        dt = sorted(times)[len(times) // 2]
+        def once_blas():                       # the same loop with the host BLAS (torch.mm) for the three GEMMs
+            t0 = time.perf_counter()
+            orc.step_blas(xs, offs, c["w"], gs, *cfg)
+            return time.perf_counter() - t0
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+        results = {}
+        for label, fn_ in (("loops", once), ("blas", once_blas)):
+            first = fn_()                      # also warms the thread pool; not counted
+            reps = max(3, min(25, int(6.0 / max(first, 1e-3))))       # about 6 s of host work per variant and configuration
+            times = sorted(fn_() for _ in range(reps))
+            results[label] = (times[len(times) // 2], reps)
+        best = min(results, key=lambda k: results[k][0])
+        dt, reps = results[best]
         cpu = {"value": round(3 * F * ns / x.shape[0] / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
                "kind": "port", "seconds": round(dt, 2),
-               "sample": "%d of %d samples of %s, forward + backward, median of %d runs, float accumulate, OpenMP" %
+               "gemm": "host BLAS through torch.mm" if best == "blas" else "plain OpenMP loops of the oracle",
+               "variants_seconds": {k: round(v[0], 3) for k, v in results.items()},
+               "sample": "%d of %d samples of %s, forward + backward, median of %d runs, float accumulate; the faster of "
+                         "the oracle's own OpenMP GEMM loops and the same per-sample loop with torch.mm for the GEMMs" %
                          (ns, x.shape[0], name, reps)}
 
     return {
@@ -240,6 +253,7 @@ def run_config(name, a):
         "ms_per_step_events": step_events, "fwd_ms_events": fwd_events, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32" if dtype == torch.float32 else "f64", "data": "synthetic",
         "config": {"workload": name + ": " + DESCR[name] +
+                               ("" if a.dtype is None else " -- computed in %s instead of its own precision" % a.dtype) +
                                ("" if a.offset_scale is None else " -- with offsets U[-%g,%g] instead of its own" % (a.offset_scale, a.offset_scale))},
         "mfma_frac_whole_step": round(value / peak, 4),
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
@@ -255,6 +269,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--offset-scale", type=float, default=None,
                     help="offsets uniform in [-s, s] instead of the configuration's own (how the rates depend on the reach of the offsets)")
+    ap.add_argument("--dtype", choices=["f32", "f64"], default=None,
+                    help="run the configuration's shapes in this precision instead of its own (f64: against the fp64 matrix peak)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic for scaling rocprof's "
                          "FETCH_SIZE / WRITE_SIZE counters)")

@@ -100,7 +100,8 @@ template <typename T> size_t workspace_need(int N, int C_in, int C_out, size_t i
     const size_t fwd_plain = (size_t)G * kV * (Mp > Mp8 ? Mp : Mp8) * Cgp * sizeof(T);
     const size_t fwd_quad = slab_bound((size_t)C_in, G, cpg, FQ) * forward_slab_elems<T>(kV, Mp8) * sizeof(T);
     const size_t fwd = (fwd_plain > fwd_quad ? fwd_plain : fwd_quad) + forward_partial_bound(N, C_out, outV, sizeof(T));
-    const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G, cpg) + 2 * align256((size_t)N * C_in * inV * sizeof(T));
+    // (+ the last whole 256-byte block of the workspace: weight bounds and the plan the device chose)
+    const size_t bwd = bwd_data_weight_bytes<T>(M, Cg, kV, G, cpg) + 2 * align256((size_t)N * C_in * inV * sizeof(T)) + 512;
     // backward_weight: two channels-last copies + one partial weight per position split (at most 256 splits,
     // and never more than about 4096 workgroups: see bww_plan)
     const int TNq = Mma<T>::TN;
@@ -293,6 +294,10 @@ static bool fused_breg2() {             // DCN_FUSED_BREG2=0: grad_output operan
 }
 static bool native16() {                // DCN_NATIVE16=0: the 16-bit forward entry points always widen to float32 first
     static const int v = [] { const char* e = getenv("DCN_NATIVE16"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
+}
+static bool global_plan() {             // DCN_GLOBAL_PLAN=0: the device never chooses the path without LDS tiling
+    static const int v = [] { const char* e = getenv("DCN_GLOBAL_PLAN"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
 }
 static bool scatter_in_lds() {
@@ -725,7 +730,13 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     T* gin_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes + tbytes);
     const int TN = Mma<T>::TN;
     const int mk = bwd_data_mk<T>(P.M);
-    float* wmax = reinterpret_cast<float*>(gin_cl);     // the channels-last gradient buffer is free on the LDS paths
+    // weight bounds (two floats) and, 64 bytes further, the plan chosen on the device: in the last whole
+    // 256-byte block of the workspace when that lies behind the two channels-last regions
+    // (dcn_workspace_bytes counts it), else at the start of the channels-last gradient, which the LDS
+    // paths do not use
+    const size_t tail_at = ws_bytes >= 256 ? (ws_bytes - 256) / 256 * 256 : 0;
+    const bool tail_words = tail_at >= wbytes + 2 * tbytes;
+    float* wmax = tail_words ? reinterpret_cast<float*>(static_cast<char*>(ws) + tail_at) : reinterpret_cast<float*>(gin_cl);
     const dim3 tgrid((P.inV + 31) / 32, (unsigned)(P.C_in + 31) / 32, (unsigned)P.N), tblock(32, 8);
 
     // 1) one kernel: scatter privatised in LDS + coordinate gradient from an LDS input halo
@@ -891,6 +902,13 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         pc.margin[0] = margins[0];
         pc.base[0] = 1.f;
         pc.far_sample = ND == 3 ? 4.5f : 1.f;       // a sample beyond the halo scatters with global atomics
+        pc.far_steep = ND == 3 ? 25.f : 0.f;        // (c4, margin 2: 3.0, 4.1, 10.4, 26.6 times the time at 49, 70, 87.5, 96 % of the samples beyond the halo)
+        // 3-D: when most samples leave even the widest halo, the path without LDS tiling (coalesced
+        // atomics on a channels-last copy; about 6.5 times the fused kernel's time on small offsets,
+        // whatever the offsets) is the cheaper one: offered as a fourth choice, its kernels launched
+        // behind the fused ones and gated on the choice (DCN_GLOBAL_PLAN=0: not offered)
+        const bool offer_global = ND == 3 && tail_words && global_plan() && (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN)) <= 0x7fffffffLL &&
+                                  P.DG <= 65535;
         int copies = 1;                             // packed weight copies
         fp[0].wt = wt;
         for (int k = 1; k < nmargins; ++k) {
@@ -913,8 +931,9 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             pc.margin[k] = pc.margin[pc.nplans - 1];
             pc.base[k] = 1e30f;
         }
-        unsigned* sel = pc.nplans > 1 ? reinterpret_cast<unsigned*>(wmax + 16) : nullptr;
+        unsigned* sel = (pc.nplans > 1 || offer_global) ? reinterpret_cast<unsigned*>(wmax + 16) : nullptr;
         pc.sel = sel;
+        pc.global_cost = offer_global ? 6.5f : 0.f;
         const size_t n_off = (size_t)P.N * P.DG * P.kV * ND * P.outV;
         // weights in the lane order of the kernel's operand loads, one slab per channel chunk; the
         // first launch clears the weight bounds and chooses the plan
@@ -983,6 +1002,28 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
                                fp[k].Ph, alts, (const unsigned*)sel, in, off, fp[k].wt, gout, (const float*)wmax, gin, goff, fp[k].csplit, (unsigned)fp[k].whole,
                                fp[k].goff_atomic);
             if (int rc = check_launch("backward_input_halo_kernel")) return rc;
+        }
+        if (offer_global) {
+            // the fourth choice: three launches that return at once unless *sel == MAX_PLANS.  They reuse
+            // the weight region and the channels-last regions, which the fused kernels no longer read then.
+            Params Pg = P;
+            Pg.tiles = (P.outV + WAVES * TN - 1) / (WAVES * TN);
+            const size_t total_w = (size_t)P.G * P.kV * P.Mp * P.Cgp, pad_w = (size_t)TAP_PAD * P.Mp * P.Cgp;
+            const size_t nelem = (size_t)P.N * P.C_in * P.inV;
+            const unsigned nb_w = (unsigned)((total_w + pad_w + 255) / 256 > 1024 ? 1024 : (total_w + pad_w + 255) / 256);
+            const unsigned nb_z = (unsigned)((nelem + 1023) / 1024 > 4096 ? 4096 : (nelem + 1023) / 1024);
+            const size_t ntiles = (size_t)P.N * ((P.C_in + 31) / 32) * ((P.inV + 31) / 32);
+            const unsigned nb_t = (unsigned)(ntiles > 16384 ? 16384 : ntiles);
+            if (trace_plans()) fprintf(stderr, "dcn backward_input_offset: path without LDS tiling offered at cost %.2f\n", pc.global_cost);
+            hipLaunchKernelGGL(global_path_prepare_kernel<T>, dim3(nb_w + nb_z + nb_t), dim3(256), 0, s, Pg, w, wt, pad_w, gin_cl, in, in_cl,
+                               nb_w, nb_z, (const unsigned*)sel, (unsigned)MAX_PLANS);
+            if (int rc = check_launch("global_path_prepare_kernel")) return rc;
+            hipLaunchKernelGGL((backward_data_kernel<T, ND, true, 0>), dim3((unsigned)Pg.N * Pg.tiles, (unsigned)P.DG), dim3(WG), 0, s, Pg,
+                               (const T*)in_cl, off, (const T*)wt, gout, gin_cl, goff, (const unsigned*)sel, (unsigned)MAX_PLANS);
+            if (int rc = check_launch("backward_data_kernel")) return rc;
+            hipLaunchKernelGGL(add_from_channels_last_kernel<T>, tgrid, tblock, 0, s, (const T*)gin_cl, gin, P.C_in, P.inV,
+                               (const unsigned*)sel, (unsigned)MAX_PLANS);
+            if (int rc = check_launch("add_from_channels_last_kernel")) return rc;
         }
         return DCN_OK;
     }

@@ -56,9 +56,19 @@ struct PlanChoice {
     int margin[MAX_PLANS];        // ascending
     float base[MAX_PLANS];        // cost of the plan when no sample leaves its halo, plan 0 = 1
     // cost added by samples beyond the halo, as a factor 1 + far_wave * P(some lane of a wavefront
-    // holds such a sample) + far_sample * P(a sample is one)
-    float far_wave, far_sample;
+    // holds such a sample) + far_sample * p + far_steep * p^8 with p = P(a sample is one): the last
+    // term for the scatter, whose global atomics spread over more and more cache lines as the offsets grow
+    float far_wave, far_sample, far_steep;
+    // > 0: the path without LDS tiling (grad-input by global atomics on a channels-last copy) is on
+    // offer as well, at this cost whatever the offsets; it is chosen (*sel = MAX_PLANS) when every
+    // halo plan costs more, i.e. when most samples would leave even the widest halo
+    float global_cost;
 };
+// A kernel of a path that the device may or may not have chosen: returns true when *gate names
+// another plan (gate == nullptr: not gated).
+__device__ inline bool gated_out(const unsigned* __restrict__ gate, unsigned want) {
+    return gate && (unsigned)__builtin_amdgcn_readfirstlane((int)*gate) != want;
+}
 // The halo fields of the chosen plan in H; false when this launch does not serve it (uniform for
 // the grid).  Kept apart from P, which stays the kernel argument: its other fields can then be
 // re-read from the argument segment wherever they are needed instead of living in registers.

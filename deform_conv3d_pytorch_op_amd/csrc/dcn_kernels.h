@@ -118,9 +118,11 @@ __device__ inline void choose_plan(const PlanChoice& pc, const S* __restrict__ o
             for (int a = 1; a < pc.nd; ++a) in_sample *= keep;
             float in_wave = in_sample;
             for (int d = 0; d < 6; ++d) in_wave *= in_wave;               // ^64
-            const float cost = pc.base[k] * (1.f + pc.far_wave * (1.f - in_wave) + pc.far_sample * (1.f - in_sample));
+            const float pf = 1.f - in_sample, pf2 = pf * pf, pf4 = pf2 * pf2;
+            const float cost = pc.base[k] * (1.f + pc.far_wave * (1.f - in_wave) + pc.far_sample * pf + pc.far_steep * pf4 * pf4);
             if (k == 0 || cost < best_cost) { best = (unsigned)k; best_cost = cost; }
         }
+        if (pc.global_cost > 0.f && best_cost > pc.global_cost) best = MAX_PLANS;      // no halo plan: the path through global memory
         *pc.sel = best;
     }
 }
@@ -404,7 +406,9 @@ __global__ void to_channels_last_kernel(const T* __restrict__ src, T* __restrict
 
 // dst[C][V] += src[V][C]
 template <typename T>
-__global__ void add_from_channels_last_kernel(const T* __restrict__ src, T* __restrict__ dst, int C, unsigned V) {
+__global__ void add_from_channels_last_kernel(const T* __restrict__ src, T* __restrict__ dst, int C, unsigned V,
+                                              const unsigned* __restrict__ gate = nullptr, unsigned gate_want = 0) {
+    if (gated_out(gate, gate_want)) return;
     __shared__ T tile[32][33];
     const size_t base = (size_t)blockIdx.z * C * V;
     const unsigned v0 = blockIdx.x * 32;
@@ -419,6 +423,60 @@ __global__ void add_from_channels_last_kernel(const T* __restrict__ src, T* __re
         const int c = c0 + i;
         const unsigned v = v0 + threadIdx.x;
         if (c < C && v < V) dst[base + (size_t)c * V + v] += tile[threadIdx.x][i];
+    }
+}
+
+// Everything the path without LDS tiling needs before its main kernel, in one launch of 256-thread
+// blocks (a launch costs microseconds also when the device has chosen another path and the blocks
+// return at once): blocks [0, nb_w) re-lay the weight as [g][tap][m][channel] with zero tap slabs
+// behind it, blocks [nb_w, nb_w + nb_z) clear the channels-last gradient, the others transpose the
+// input into its channels-last copy, 32 x 32 tiles through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void global_path_prepare_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wt, size_t wt_pad,
+                                                                  T* __restrict__ gin_cl, const T* __restrict__ in, T* __restrict__ in_cl,
+                                                                  unsigned nb_w, unsigned nb_z, const unsigned* __restrict__ gate,
+                                                                  unsigned gate_want) {
+    if (gated_out(gate, gate_want)) return;
+    const unsigned b = blockIdx.x;
+    if (b < nb_w) {
+        const size_t total = (size_t)P.G * P.kV * P.Mp * P.Cgp;
+        for (size_t i = (size_t)b * 256 + threadIdx.x; i < total + wt_pad; i += (size_t)nb_w * 256) {
+            T v = 0;
+            if (i < total) {
+                const int cl = i % P.Cgp;
+                size_t t = i / P.Cgp;
+                const int m = t % P.Mp;
+                t /= P.Mp;
+                const int tap = t % P.kV, g = t / P.kV;
+                if (m < P.M && cl < P.Cg) v = W[(((size_t)g * P.M + m) * P.Cg + cl) * P.kV + tap];
+            }
+            Wt[i] = v;
+        }
+        return;
+    }
+    const size_t nelem = (size_t)P.N * P.C_in * P.inV;
+    if (b < nb_w + nb_z) {
+        for (size_t i = (size_t)(b - nb_w) * 256 + threadIdx.x; i < nelem; i += (size_t)nb_z * 256) gin_cl[i] = 0;
+        return;
+    }
+    __shared__ T tile[32][33];
+    const unsigned tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const unsigned vt = (P.inV + 31) / 32, ct = ((unsigned)P.C_in + 31) / 32;
+    const size_t ntiles = (size_t)P.N * ct * vt;
+    const unsigned nb_t = gridDim.x - nb_w - nb_z;
+    for (size_t tno = b - nb_w - nb_z; tno < ntiles; tno += nb_t) {
+        const unsigned v0 = (unsigned)(tno % vt) * 32, c0 = (unsigned)((tno / vt) % ct) * 32;
+        const size_t base = (tno / vt / ct) * (size_t)P.C_in * P.inV;
+        __syncthreads();
+        for (unsigned i = ty; i < 32; i += 8) {
+            const unsigned c = c0 + i, v = v0 + tx;
+            if (c < (unsigned)P.C_in && v < P.inV) tile[i][tx] = in[base + (size_t)c * P.inV + v];
+        }
+        __syncthreads();
+        for (unsigned i = ty; i < 32; i += 8) {
+            const unsigned v = v0 + i, c = c0 + tx;
+            if (c < (unsigned)P.C_in && v < P.inV) in_cl[base + (size_t)v * P.C_in + c] = tile[tx][i];
+        }
     }
 }
 
@@ -507,7 +565,9 @@ template <typename T, int ND, bool SCATTER, int MK>
 __global__ __launch_bounds__(WG) void backward_data_kernel(Params P, const T* __restrict__ in_cl,
                                                            const T* __restrict__ off, const T* __restrict__ Wt,
                                                            const T* __restrict__ gout, T* __restrict__ gin_cl,
-                                                           T* __restrict__ goff) {
+                                                           T* __restrict__ goff, const unsigned* __restrict__ gate = nullptr,
+                                                           unsigned gate_want = 0) {
+    if (gated_out(gate, gate_want)) return;
     using MM = Mma<T>;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
     __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // corner voxel index * C_in

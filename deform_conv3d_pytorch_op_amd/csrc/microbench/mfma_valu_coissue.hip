@@ -12,7 +12,8 @@ typedef float f4v __attribute__((ext_vector_type(4)));
 typedef double d4v __attribute__((ext_vector_type(4)));
 
 // VK: 0 v_fma_f32, 1 v_add_u32, 2 v_cndmask_b32, 3 v_fma_f64, 4 v_cvt_f64_f32, 5 v_mul_f32, 6 v_lshl_add_u32, 7 v_cmp_lt_f32, 8 v_add_f32, 9 v_cvt_i32_f32, 10 v_mad_u32_u24, 11 v_med3_f32, 12 v_floor_f32
-// MK: 0 none, 1 32x32x2 f32, 2 16x16x4 f32, 3 16x16x4 f64
+// MK: 0 none, 1 32x32x2 f32, 2 16x16x4 f32, 3 16x16x4 f64, 4 32x32x8 bf16, 5 32x32x16 bf16 (both accumulate in float),
+//     6 32x32x16 bf16 with the accumulator in AGPRs, 7 32x32x2 f32 with the accumulator in AGPRs
 template <int MK, int NM, int VK, int NV, int NT>
 __global__ __launch_bounds__(NT) void k(int iters, float* out) {
     f16v acc0 = {0}, acc1 = {0};
@@ -57,6 +58,22 @@ __global__ __launch_bounds__(NT) void k(int iters, float* out) {
                     if (i & 1) asm volatile("v_mfma_f64_16x16x4_f64 %0, %1, %2, %0" : "+v"(c1) : "v"(ad), "v"(bd));
                     else       asm volatile("v_mfma_f64_16x16x4_f64 %0, %1, %2, %0" : "+v"(c0) : "v"(ad), "v"(bd));
                 }
+                if (MK == 4) {          // four bfloat16 per lane and operand: a 64-bit register pair each
+                    if (i & 1) asm volatile("v_mfma_f32_32x32x8_bf16 %0, %1, %2, %0" : "+v"(acc1) : "v"(ad), "v"(bd));
+                    else       asm volatile("v_mfma_f32_32x32x8_bf16 %0, %1, %2, %0" : "+v"(acc0) : "v"(ad), "v"(bd));
+                }
+                if (MK == 5) {          // eight bfloat16 per lane and operand: four registers each
+                    if (i & 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc1) : "v"(b0), "v"(b1));
+                    else       asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc0) : "v"(b0), "v"(b1));
+                }
+                if (MK == 6) {
+                    if (i & 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc1) : "v"(b0), "v"(b1));
+                    else       asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc0) : "v"(b0), "v"(b1));
+                }
+                if (MK == 7) {
+                    if (i & 1) asm volatile("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(acc1) : "v"(a), "v"(b));
+                    else       asm volatile("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(acc0) : "v"(a), "v"(b));
+                }
             }
         }
     }
@@ -96,6 +113,11 @@ int main() {
     CK(hipMalloc(&d_out, 64));
     rows<0>(); rows<1>(); rows<3>(); rows<4>(); rows<5>(); rows<6>(); rows<7>(); rows<8>(); rows<9>(); rows<10>(); rows<11>(); rows<12>();
     row<2, 16, 0, 512>("mfma 16x16x4 f32"); row<2, 16, 0, 1024>("mfma 16x16x4 f32"); row<2, 16, 1, 1024>("mfma 16x16x4 f32");
+    // 16-bit matrix instructions (f32 accumulation) beside vector work: do they share the issue port too?
+    row<4, 8, 0, 512>("mfma 32x32x8 bf16"); row<4, 8, 0, 1024>("mfma 32x32x8 bf16"); row<4, 8, 1, 1024>("mfma 32x32x8 bf16"); row<4, 8, 9, 1024>("mfma 32x32x8 bf16");
+    row<5, 8, 0, 512>("mfma 32x32x16bf16"); row<5, 8, 0, 1024>("mfma 32x32x16bf16"); row<5, 8, 1, 1024>("mfma 32x32x16bf16"); row<5, 8, 9, 1024>("mfma 32x32x16bf16");
+    row<6, 8, 0, 512>("32x32x16bf16 agpr"); row<6, 8, 0, 1024>("32x32x16bf16 agpr"); row<6, 8, 1, 1024>("32x32x16bf16 agpr");
+    row<7, 8, 0, 512>("32x32x2 f32 agpr"); row<7, 8, 0, 1024>("32x32x2 f32 agpr");
     row<3, 16, 0, 512>("mfma 16x16x4 f64"); row<3, 16, 0, 1024>("mfma 16x16x4 f64"); row<3, 16, 1, 1024>("mfma 16x16x4 f64"); row<3, 16, 3, 1024>("mfma 16x16x4 f64");
     return 0;
 }

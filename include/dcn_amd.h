@@ -69,7 +69,9 @@ const char *dcn_last_error(void);   /* message of the last failing call on this 
  * one word in which the device records which of the planned LDS halo sizes it chose for the call
  * from the offsets (so two calls that overlap in time need a workspace each; the forward calls
  * keep it as a 32-bit index, 0 = the narrowest halo, at byte offset (workspace_bytes - 256) rounded
- * down to a multiple of 256). */
+ * down to a multiple of 256, the backward_input_offset calls 64 bytes further; there the value 3
+ * means that the device took the path without LDS tiling, which it does for a 3-D layer when most
+ * samples would leave even the widest halo). */
 size_t dcn_workspace_bytes(int elem_size, int batch, int input_c, int output_c, size_t input_volume,
                            size_t output_volume, int kernel_volume, int group);
 /* The same for a known number of channels per deformable group (the reference's

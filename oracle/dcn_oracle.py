@@ -152,3 +152,39 @@ def col2im_offset(col, im, off, weight_shape, stride, padding, dilation, channel
     goff = torch.zeros_like(off)
     lib().dcn_oracle_col2im_offset(_dt(col), geom, _p(col), _p(im), _p(off), _p(goff))
     return goff
+
+
+# --- the reference's sequencing with the host BLAS for its three GEMMs ------------------------
+# deform3d/lib/deform_conv3d_cuda.cpp:105-158 (forward), :186-253 (backward to input and offset) and
+# :278-330 (backward to weight) loop over the samples, build the column buffer of a sample with
+# deformable_im2col, and call one cuBLAS GEMM per convolution group.  This is that loop with
+# torch.mm (the host BLAS) in the place of cuBLAS and the oracle's C++ stages for the rest; the
+# benchmark times it as the CPU baseline.
+
+def step_blas(inputs, offset, weight, grad_output, stride=1, padding=0, dilation=1, channel_per_group=1, group=1):
+    """Forward + backward of the reference algorithm on the host: (output, grad_input, grad_offset, grad_weight)."""
+    N, C_in, C_out = inputs.shape[0], inputs.shape[1], weight.shape[0]
+    wshape = tuple(weight.shape[2:])
+    kV = weight[0, 0].numel()
+    M, Kg = C_out // group, (C_in // group) * kV
+    w2 = weight.reshape(group, M, Kg)
+    out = gin = goff = None
+    gw = torch.zeros_like(w2)
+    for n in range(N):
+        col = im2col(inputs[n], offset[n], wshape, stride, padding, dilation, channel_per_group)      # [C_in*kV, outV]
+        outV = col.shape[1]
+        if out is None:
+            outs = tuple(grad_output.shape[2:])
+            out = inputs.new_empty((N, C_out) + outs)
+            gin, goff = torch.zeros_like(inputs), torch.zeros_like(offset)
+        colg = col.view(group, Kg, outV)
+        go = grad_output[n].reshape(group, M, outV)
+        gcol = torch.empty_like(colg)
+        for g in range(group):
+            out[n].view(group, M, outV)[g] = torch.mm(w2[g], colg[g])              # G1
+            gcol[g] = torch.mm(w2[g].t(), go[g])                                   # G2
+            gw[g] += torch.mm(go[g], colg[g].t())                                  # G3 (the reference rebuilds the columns first)
+        gcol = gcol.view(C_in * kV, outV)
+        gin[n] = col2im_input(gcol, offset[n], inputs.shape[1:], wshape, stride, padding, dilation, channel_per_group)
+        goff[n] = col2im_offset(gcol, inputs[n], offset[n], wshape, stride, padding, dilation, channel_per_group)
+    return out, gin, goff, gw.view_as(weight)

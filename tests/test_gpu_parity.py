@@ -698,3 +698,41 @@ def test_heavy_tailed_grad_output_keeps_small_gradients(name):
     assert excess <= eps, "grad_input: %.3e of max|ref| beyond 1e-3 |ref|" % excess
     for nm, gt, wt in zip(("output", "grad_input", "grad_offset", "grad_weight"), got, want):
         assert rel_err(gt, wt) <= TOL[torch.float32]["fwd" if nm == "output" else "grad"], nm
+
+
+def test_backward_plan_follows_the_offsets_up_to_the_path_without_lds():
+    """backward_input_offset records the plan the device chose 64 bytes into the last whole 256-byte
+    block of its workspace (include/dcn_amd.h): 0 for offsets within +-1, a wider halo for +-2.6, and 3
+    -- the path without LDS tiling, coalesced atomics on a channels-last copy -- when the offsets
+    (+-9) throw most samples beyond the widest halo.  The gradients agree with the oracle whichever
+    path runs, and grad_input is accumulated into by all of them."""
+    if os.environ.get("DCN_HALO_MARGIN") or os.environ.get("DCN_ADAPTIVE_MARGIN") == "0" or \
+            os.environ.get("DCN_GLOBAL_PLAN") == "0" or os.environ.get("DCN_SCATTER") or os.environ.get("DCN_COORD"):
+        pytest.skip("the choice is switched off by a knob")
+    from deform_conv3d_pytorch_op_amd import _lib
+    from deform_conv3d_pytorch_op_amd.functions import _geom
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    spec = (3, 2, 16, 16, (8, 16, 24), 3, 1, 1, 1, 8, 1)
+    chosen = {}
+    for label, scale in (("narrow", 1.0), ("wide", 2.6), ("huge", 9.0)):
+        print("backward plan", label, flush=True)
+        c = make_case(*spec, scale, dtype=torch.float32, seed=22, bias=False)
+        x, off, w, gout = (c[k].to(dev) for k in ("x", "off", "w", "gout"))
+        geom = _geom(3, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+        nbytes = L.dcn_workspace_bytes_for(4, x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]), math.prod(c["outs"]),
+                                           math.prod(c["k"]), c["groups"], c["cpg"])
+        ws = torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=dev)
+        gin = torch.ones_like(x)                        # accumulated into
+        goff = torch.full_like(off, 7.0)                # overwritten
+        rc = L.dcn3d_backward_input_offset_f32(x.data_ptr(), w.data_ptr(), off.data_ptr(), gout.data_ptr(), gin.data_ptr(),
+                                               goff.data_ptr(), *geom, ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, L.dcn_last_error()
+        torch.cuda.synchronize()
+        at = (nbytes - 256) // 256 * 256 + 64
+        chosen[label] = int.from_bytes(bytes(ws[at:at + 4].cpu().tolist()), "little")
+        want_gin, want_goff, _, _ = orc.backward(c["x"], c["off"], c["w"], c["gout"], None, c["stride"], c["pad"], c["dil"],
+                                                 c["cpg"], c["groups"])
+        assert rel_err(gin - 1.0, want_gin) < TOL[torch.float32]["grad"], label
+        assert rel_err(goff, want_goff) < TOL[torch.float32]["grad"], label
+    assert chosen["narrow"] == 0 and chosen["wide"] in (1, 2) and chosen["huge"] == 3, chosen

@@ -14,6 +14,7 @@ import torch.nn.functional as F
 
 from oracle import dcn_oracle as orc
 from tests import composite_ref as comp
+from tests.cases import SMALL_CASES, make_case
 
 torch.manual_seed(0)
 
@@ -324,3 +325,16 @@ def test_float_oracle_close_to_double():
         assert d < 1e-4
         for a, b in zip(oracle_bwd(c32, acc64), oracle_bwd(c64r)):
             assert (a.double() - b).abs().max() < 1e-3
+
+
+def test_blas_sequencing_equals_the_oracle_loops():
+    """The reference's per-sample loop with torch.mm for its three GEMMs (the timed CPU baseline) gives
+    what the oracle's own loops give."""
+    for name in ("3d_basic", "2d_c3_like", "3d_mixed"):
+        c = make_case(*SMALL_CASES[name], dtype=torch.float64, seed=21, bias=False)
+        cfg = (c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
+        out, gin, goff, gw = orc.step_blas(c["x"], c["off"], c["w"], c["gout"], *cfg)
+        want_out = orc.forward(c["x"], c["off"], c["w"], None, *cfg)
+        want = orc.backward(c["x"], c["off"], c["w"], c["gout"], None, *cfg)
+        for got, ref in ((out, want_out), (gin, want[0]), (goff, want[1]), (gw, want[2])):
+            assert (got - ref).abs().max().item() <= 1e-12 * max(1.0, ref.abs().max().item()), name
