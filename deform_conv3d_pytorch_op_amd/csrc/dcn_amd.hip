@@ -57,9 +57,9 @@ size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 constexpr int TAP_PAD = 8;      // zero tap slabs behind the last group: an MFMA pass may start up to 7 taps before the end
 // Elements of the per-chunk weight slabs of the fused backward kernel (pack_weight_kernel, chunks of
 // `cch` channels) for `slabs` slabs.
-template <typename T> size_t packed_weight_elems(int M, int kV, size_t slabs, int cch) {
-    const int KL = Mma<T>::KL, TP = Mma<T>::TN / cch;
-    return slabs * ((kV + TP - 1) / TP) * (size_t)(((M + KL - 1) / KL + 15) / 16 * 16) * 64;
+template <typename T, typename S = T> size_t packed_weight_elems(int M, int kV, size_t slabs, int cch) {
+    const int TP = Mma<T>::TN / cch;
+    return slabs * ((kV + TP - 1) / TP) * (size_t)gcol_slab_steps<T, S>(M) * 64 * (std::is_same<S, T>::value ? 1 : 4);
 }
 // Upper bound of chunk_slot<cch>(cpg, Cg, c) + 1 over the channels: the slabs a per-chunk weight
 // layout occupies.  cpg = 0: the channels per deformable group are not known (the first workspace
@@ -709,9 +709,15 @@ int weight_bounds(const Params& P, const T* w, float* out, hipStream_t s) {
 }
 
 constexpr unsigned FLAG_INPUT_ONLY = 0x100u;     // internal: see backward_input_offset
-template <typename T, int ND>
-int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* off, const T* gout, T* gin,
-                          T* goff, void* ws, size_t ws_bytes, hipStream_t s, unsigned flags = 0) {
+// S = T: the float32 / float64 operator.  S = Bf16 / Fp16 (T = float): input, weight, offset and
+// grad_output are in that storage format (the gradients are float), and only the fused kernel with
+// its grad_output operand in registers serves them, on the 16-bit matrix instructions; where it
+// cannot, *declined is set and nothing is launched: the caller then widens the tensors and runs the
+// float32 operator.
+template <typename T, int ND, typename S = T>
+int backward_input_offset(const Geometry& g, const S* in, const S* w, const S* off, const S* gout, T* gin,
+                          T* goff, void* ws, size_t ws_bytes, hipStream_t s, unsigned flags = 0, bool* declined = nullptr) {
+    constexpr bool S16 = !std::is_same<S, T>::value;
     Params P;
     if (int rc = validate(g, P)) return rc;
     if (flags & ~(unsigned)(DCN_FLAG_OOB_OFFSET_GRAD_ZERO | FLAG_INPUT_ONLY)) return fail(DCN_E_ARGUMENT, "unknown flag");
@@ -725,7 +731,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     const size_t wbytes = bwd_data_weight_bytes<T>(P.M, P.Cg, P.kV, P.G, P.cpg);
     const size_t tbytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(T));
     if (!ws || ws_bytes < wbytes + 2 * tbytes) return fail(DCN_E_WORKSPACE, "workspace too small");
-    T* wt = static_cast<T*>(ws);
+    S* wt = static_cast<S*>(ws);
     T* in_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes);
     T* gin_cl = reinterpret_cast<T*>(static_cast<char*>(ws) + wbytes + tbytes);
     const int TN = Mma<T>::TN;
@@ -746,7 +752,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     // halo) where only that fits, e.g. under stride 2.
     constexpr int FUSED_HS = sizeof(T) == 4 ? 2720 : 2112;
     constexpr int FUSED_HS8 = 2016;     // plane stride of the 8-channel float instantiation with compile-time halo extents
-    using Kern = void (*)(Params, PlanSet, const unsigned*, const T*, const T*, const T*, const T*, const float*, T*, T*, int, unsigned, int);
+    using Kern = void (*)(Params, PlanSet, const unsigned*, const S*, const S*, const S*, const S*, const float*, T*, T*, int, unsigned, int);
     struct FusedPlan {
         Params Ph;
         Kern kern;
@@ -755,7 +761,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         bool wide;
         long long whole, items, slots;
         size_t lds;
-        const T* wt;
+        const S* wt;
     };
     const int seg = P.cpg < P.Cg ? P.cpg : P.Cg;
     // Plans the fused kernel for a halo of margin m; false when none of its shapes fits.
@@ -806,19 +812,21 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             if (fixed && !eight) Ph.hstride = FUSED_HS;
             // grad_output operand held in registers when its reduction steps fit: 32 per pass
             // (M <= 64 float, 128 double with 4-channel chunks)
-            const int ksteps = (P.M + Mma<T>::KL - 1) / Mma<T>::KL;
-            const bool wide = eight && !sixteen && pair && ksteps <= 32;                             // the kernel's WIDE
+            // (16-bit storage: a reduction step takes 8 output channels and an operand batch half as many steps)
+            const int KS = GcolGemm<T, S>::KS, halve = S16 ? 2 : 1;
+            const int ksteps = (P.M + KS - 1) / KS;
+            const bool wide = eight && !sixteen && pair && ksteps <= 32 / halve;                     // the kernel's WIDE
             const int slot_regs = (wide || sixteen) ? 8 : (Mma<T>::row(1, 0) - Mma<T>::row(0, 0) == 1) ? 4 : cch / 4;      // the kernel's RPS
-            const bool breg = ksteps <= Mma<T>::NACC / slot_regs * ((wide || sixteen) ? 16 : 8);
-            // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels
-            const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 && fused_breg2();
+            const bool breg = ksteps <= Mma<T>::NACC / slot_regs * ((wide || sixteen) ? 16 : 8) / halve;
+            // float, 4-channel chunks: a second set of 32 registers takes the operand of up to 128 output channels (16-bit: 256)
+            const bool breg2 = sizeof(T) == 4 && !eight && !breg && ksteps <= 64 / halve && fused_breg2();
             special = ND == 3 && eight && !sixteen && pair && wide && breg && fused_fixed_stride() && Ph.hext[1] == 14 && Ph.hext[2] == 14 &&
                       Ph.hstride <= FUSED_HS8;
             if (special) Ph.hstride = FUSED_HS8;
             const size_t lds = (size_t)cch * Ph.hstride * chb + tables;
             Kern kern = nullptr;
-#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, BREG_, HS_, NW_, true, PAIR_>
-#define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2>
+#define DCN_FUSED_C(CCH_, BREG_, HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, CCH_, true, (BREG_) || S16, HS_, NW_, true, PAIR_, 1, 0, 0, S>
+#define DCN_FUSED_B2(HS_, NW_, PAIR_) backward_input_halo_kernel<T, ND, 4, true, true, HS_, NW_, true, PAIR_, 2, 0, 0, S>
             auto pick = [&](auto pair_tag) {
                 constexpr bool PR = decltype(pair_tag)::value;
                 if (sixteen) {
@@ -828,7 +836,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
                     // the halo of a 3x3x3 kernel at stride 1 and margin 2 under the default block of positions:
                     // inner extents 14 x 14 and the plane stride fixed at compile time
                     if constexpr (ND == 3 && PR && sizeof(T) == 4) {
-                        if (special) kern = backward_input_halo_kernel<T, ND, 8, true, true, FUSED_HS8, 8, true, true, 1, 14, 14>;
+                        if (special) kern = backward_input_halo_kernel<T, ND, 8, true, true, FUSED_HS8, 8, true, true, 1, 14, 14, S>;
                     }
                 } else if (breg2) {
                     if constexpr (sizeof(T) == 4) {
@@ -848,6 +856,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
 #undef DCN_FUSED_B2
 #undef DCN_FUSED_C
             if (!kern) continue;
+            if (S16 && !breg && !breg2) continue;       // 16-bit operands come from registers only
             // Work items are (tile, deformable group) pairs, each a run of nchunks channel chunks.  `slots`
             // workgroups run at once, so the items take whole rounds plus a partly filled last one.  Either
             // every item is split over 1, 2 or 4 workgroups (workgroup cz takes every csplit-th chunk), or
@@ -892,6 +901,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     FusedPlan fp[MAX_PLANS];
     int margins[MAX_PLANS];
     const int nmargins = plan_margins(ND, margins);
+    if (S16 && !(scatter_in_lds() && fused_coord() && !input_only && native16())) {
+        if (declined) *declined = true;
+        return DCN_OK;
+    }
     if (scatter_in_lds() && fused_coord() && !input_only && plan_fused(margins[0], fp[0])) {
         // Wider halos for offsets that reach further; the choice is made on the device, see
         // PlanChoice.  A plan whose weights want another lane order gets a packed copy of its own in
@@ -907,7 +920,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         // atomics on a channels-last copy; about 6.5 times the fused kernel's time on small offsets,
         // whatever the offsets) is the cheaper one: offered as a fourth choice, its kernels launched
         // behind the fused ones and gated on the choice (DCN_GLOBAL_PLAN=0: not offered)
-        const bool offer_global = ND == 3 && tail_words && global_plan() && (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN)) <= 0x7fffffffLL &&
+        const bool offer_global = !S16 && ND == 3 && tail_words && global_plan() && (long long)P.N * ((P.outV + WAVES * TN - 1) / (WAVES * TN)) <= 0x7fffffffLL &&
                                   P.DG <= 65535;
         int copies = 1;                             // packed weight copies
         fp[0].wt = wt;
@@ -918,7 +931,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
                 if (fp[e].cch == c.cch && fp[e].wide == c.wide) c.wt = fp[e].wt;
             if (!c.wt) {
                 if ((size_t)copies * wbytes > tbytes) continue;
-                c.wt = reinterpret_cast<const T*>(reinterpret_cast<const char*>(in_cl) + (size_t)(copies - 1) * wbytes);
+                c.wt = reinterpret_cast<const S*>(reinterpret_cast<const char*>(in_cl) + (size_t)(copies - 1) * wbytes);
                 ++copies;
             }
             pc.margin[pc.nplans] = margins[k];
@@ -942,23 +955,23 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
             for (int e = 0; e < k; ++e) packed = packed || fp[e].wt == fp[k].wt;
             if (packed) continue;
             const bool sixteen = fp[k].cch == 16, eight = fp[k].cch == 8, wide = fp[k].wide;
-            const size_t total = packed_weight_elems<T>(P.M, P.kV, (size_t)(sixteen ? chunk_candidates<16>(P.cpg, P.Cg, P.C_in)
+            const size_t total = packed_weight_elems<T, S>(P.M, P.kV, (size_t)(sixteen ? chunk_candidates<16>(P.cpg, P.Cg, P.C_in)
                                                                             : eight ? chunk_candidates<8>(P.cpg, P.Cg, P.C_in)
                                                                                     : chunk_candidates<4>(P.cpg, P.Cg, P.C_in)), fp[k].cch);
             const unsigned blocks = (unsigned)((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
             PlanChoice pk = pc;
             if (k > 0) pk.sel = nullptr;
             float* bounds = k == 0 ? wmax : nullptr;
-            T* dst = const_cast<T*>(fp[k].wt);
+            S* dst = const_cast<S*>(fp[k].wt);
             const dim3 pgrid(blocks + (pk.sel ? 1 : 0));
             // (wide: row order that leaves the eight channels of a tap in one lane)
-            if (sixteen) hipLaunchKernelGGL((pack_weight_kernel<T, 16>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
-            else if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
-            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
-            else hipLaunchKernelGGL((pack_weight_kernel<T, 4>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            if (sixteen) hipLaunchKernelGGL((pack_weight_kernel<T, 16, false, S>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            else if (wide) hipLaunchKernelGGL((pack_weight_kernel<T, 8, true, S>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            else if (eight) hipLaunchKernelGGL((pack_weight_kernel<T, 8, false, S>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
+            else hipLaunchKernelGGL((pack_weight_kernel<T, 4, false, S>), pgrid, dim3(256), 0, s, P, w, dst, bounds, pk, off, n_off);
             if (int rc = check_launch("pack_weight_kernel")) return rc;
         }
-        if (int rc = weight_bounds<T>(P, w, wmax, s)) return rc;
+        if (int rc = weight_bounds<S>(P, w, wmax, s)) return rc;
         bool any_atomic = false;
         for (int k = 0; k < pc.nplans; ++k) any_atomic = any_atomic || fp[k].zero_goff;
         if (any_atomic) {
@@ -1003,7 +1016,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
                                fp[k].goff_atomic);
             if (int rc = check_launch("backward_input_halo_kernel")) return rc;
         }
-        if (offer_global) {
+        if constexpr (!S16) if (offer_global) {
             // the fourth choice: three launches that return at once unless *sel == MAX_PLANS.  They reuse
             // the weight region and the channels-last regions, which the fused kernels no longer read then.
             Params Pg = P;
@@ -1027,6 +1040,10 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
         }
         return DCN_OK;
     }
+    if constexpr (S16) {
+        if (declined) *declined = true;
+        return DCN_OK;
+    } else {
 
     // 2) grad_offset from the channels-last kernel, grad_input from the LDS-privatised scatter
     if (int rc = relayout<T>(P, w, wt, 1, s)) return rc;
@@ -1092,6 +1109,7 @@ int backward_input_offset(const Geometry& g, const T* in, const T* w, const T* o
     if (int rc = check_launch("backward_data_kernel")) return rc;
     hipLaunchKernelGGL(add_from_channels_last_kernel<T>, tgrid, tblock, 0, s, gin_cl, gin, P.C_in, P.inV);
     return check_launch("add_from_channels_last_kernel");
+    }
 }
 
 // Plan of backward_weight: channel tiles, m chunks and the number of position splits.
@@ -1280,12 +1298,22 @@ int backward_input_offset16(const Geometry& g, const S* in, const S* w, const S*
     Carver c{static_cast<char*>(ws), ws ? ws_bytes : 0};
     float *fin = c.take(z.in), *fw = c.take(z.w), *foff = c.take(z.off), *fgout = c.take(z.out), *fgin = c.take(z.in), *fgoff = c.take(z.off);
     if (!fin || !fw || !foff || !fgout || !fgin || !fgoff) return fail(DCN_E_WORKSPACE, "workspace too small");
-    if (int rc = widen(in, fin, z.in, s)) return rc;
-    if (int rc = widen(w, fw, z.w, s)) return rc;
-    if (int rc = widen(off, foff, z.off, s)) return rc;
-    if (int rc = widen(gout, fgout, z.out, s)) return rc;
     if (int rc = widen(gin, fgin, z.in, s)) return rc;            // grad_input is accumulated into
-    if (int rc = backward_input_offset<float, ND>(g, fin, fw, foff, fgout, fgin, fgoff, c.p, c.left, s)) return rc;
+    // the fused kernel reads the 16-bit tensors itself and forms the grad columns with 16-bit matrix
+    // instructions (the products of 16-bit values are exact in float, so the results are those of the
+    // float32 kernel up to the order of the sums); the gradients leave it as float and are rounded once
+    bool declined = true;
+    if (native16()) {
+        declined = false;
+        if (int rc = backward_input_offset<float, ND, S>(g, in, w, off, gout, fgin, fgoff, c.p, c.left, s, 0, &declined)) return rc;
+    }
+    if (declined) {
+        if (int rc = widen(in, fin, z.in, s)) return rc;
+        if (int rc = widen(w, fw, z.w, s)) return rc;
+        if (int rc = widen(off, foff, z.off, s)) return rc;
+        if (int rc = widen(gout, fgout, z.out, s)) return rc;
+        if (int rc = backward_input_offset<float, ND>(g, fin, fw, foff, fgout, fgin, fgoff, c.p, c.left, s)) return rc;
+    }
     if (int rc = narrow(fgin, gin, z.in, s)) return rc;
     return narrow(fgoff, goff, z.off, s);
 }
@@ -1341,7 +1369,7 @@ int conv2d_backward_input(Geometry g, const T* w, const T* gout, T* gin, void* w
     g.cpg = g.C_in;
     T *off, *scratch; void* rest; size_t rest_bytes;
     if (int rc = conv2d_offsets<T>(g, ws, ws_bytes, s, &off, &scratch, &rest, &rest_bytes)) return rc;
-    return backward_input_offset<T, 2>(g, nullptr, w, off, gout, gin, scratch, rest, rest_bytes, s, FLAG_INPUT_ONLY);
+    return backward_input_offset<T, 2>(g, static_cast<const T*>(nullptr), w, static_cast<const T*>(off), gout, gin, scratch, rest, rest_bytes, s, FLAG_INPUT_ONLY);
 }
 template <typename T>
 int conv2d_backward_weight(Geometry g, const T* in, const T* gout, T* gw, void* ws, size_t ws_bytes, hipStream_t s) {

@@ -22,36 +22,6 @@ namespace dcn {
 
 constexpr int FQ = 4;              // channels per group: one wide LDS read per corner
 
-// Storage format of the tensors in global memory.  float / double: the arithmetic type itself.
-// Bf16 / Fp16: 16-bit storage, float arithmetic; the sampled columns and the weights then meet in
-// v_mfma_f32_32x32x8_bf16 / _f16 (float accumulation), a quarter of the matrix instructions.
-template <typename S> struct Store { static __device__ inline S ld(S v) { return v; } static __device__ inline S st(S v) { return v; } };
-template <> struct Store<Bf16> {
-    static __device__ inline float ld(Bf16 v) { return Bf16::widen(v); }
-    static __device__ inline Bf16 st(float v) { return Bf16::narrow(v); }
-};
-template <> struct Store<Fp16> {
-    static __device__ inline float ld(Fp16 v) { return Fp16::widen(v); }
-    static __device__ inline Fp16 st(float v) { return Fp16::narrow(v); }
-};
-typedef short Short4 __attribute__((ext_vector_type(4)));
-typedef _Float16 Half4 __attribute__((ext_vector_type(4)));
-typedef __bf16 Bfloat4 __attribute__((ext_vector_type(4)));
-template <typename S> struct Mma16;
-template <> struct Mma16<Bf16> {
-    typedef Short4 Vec;
-    static __device__ inline Vec pack(const float v[4]) {
-        const Bfloat4 b = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};      // round to nearest even
-        return __builtin_bit_cast(Short4, b);
-    }
-    static __device__ inline Mma<float>::Acc mma(Vec a, Vec b, Mma<float>::Acc c) { return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a, b, c, 0, 0, 0); }
-};
-template <> struct Mma16<Fp16> {
-    typedef Half4 Vec;
-    static __device__ inline Vec pack(const float v[4]) { return Vec{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]}; }
-    static __device__ inline Mma<float>::Acc mma(Vec a, Vec b, Mma<float>::Acc c) { return __builtin_amdgcn_mfma_f32_32x32x8f16(a, b, c, 0, 0, 0); }
-};
-
 // Weights of the forward kernel: one slab per group of four channels (groups start at the first
 // channel of a segment -- the channels shared by one deformable group and one convolution group --
 // and every fourth after it), in the order the lanes consume them:

@@ -9,12 +9,74 @@
 #pragma once
 #include "dcn_device.h"
 #include <limits>
+#include <type_traits>
 
 
 namespace dcn {
 
 constexpr int WG = 256;            // 4 wavefronts
 constexpr int WAVES = WG / 64;
+
+// 16-bit storage formats of the mixed-precision entry points: the tensors are widened to float
+// (exactly) before the float32 kernels run and the results are rounded once, to nearest even.
+struct Bf16 {       // bfloat16: the upper half of a float
+    unsigned short bits;
+    __device__ static inline float widen(Bf16 v) { return __uint_as_float((unsigned)v.bits << 16); }
+    __device__ static inline Bf16 narrow(float f) {
+        const unsigned u = __float_as_uint(f);
+        Bf16 r;
+        if ((u & 0x7fffffffu) > 0x7f800000u) r.bits = (unsigned short)((u >> 16) | 0x40u);      // NaN stays NaN
+        else r.bits = (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);                  // Inf and overflow to Inf included
+        return r;
+    }
+};
+struct Fp16 {       // IEEE binary16
+    _Float16 v;
+    __device__ static inline float widen(Fp16 x) { return (float)x.v; }
+    __device__ static inline Fp16 narrow(float f) { Fp16 r; r.v = (_Float16)f; return r; }
+};
+__device__ inline float offset_value(Bf16 v) { return Bf16::widen(v); }
+__device__ inline float offset_value(Fp16 v) { return Fp16::widen(v); }
+
+// Storage format of the tensors in global memory.  float / double: the arithmetic type itself.
+// Bf16 / Fp16: 16-bit storage, float arithmetic; the sampled columns and the weights then meet in
+// v_mfma_f32_32x32x8_bf16 / _f16 (float accumulation), a quarter of the matrix instructions.
+template <typename S> struct Store { static __device__ inline S ld(S v) { return v; } static __device__ inline S st(S v) { return v; } };
+template <> struct Store<Bf16> {
+    static __device__ inline float ld(Bf16 v) { return Bf16::widen(v); }
+    static __device__ inline Bf16 st(float v) { return Bf16::narrow(v); }
+};
+template <> struct Store<Fp16> {
+    static __device__ inline float ld(Fp16 v) { return Fp16::widen(v); }
+    static __device__ inline Fp16 st(float v) { return Fp16::narrow(v); }
+};
+typedef short Short4 __attribute__((ext_vector_type(4)));
+typedef _Float16 Half4 __attribute__((ext_vector_type(4)));
+typedef __bf16 Bfloat4 __attribute__((ext_vector_type(4)));
+template <typename S> struct Mma16;
+template <> struct Mma16<Bf16> {
+    typedef Short4 Vec;
+    static __device__ inline Vec pack(const float v[4]) {
+        const Bfloat4 b = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};      // round to nearest even
+        return __builtin_bit_cast(Short4, b);
+    }
+    static __device__ inline Mma<float>::Acc mma(Vec a, Vec b, Mma<float>::Acc c) { return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a, b, c, 0, 0, 0); }
+};
+template <> struct Mma16<Fp16> {
+    typedef Half4 Vec;
+    static __device__ inline Vec pack(const float v[4]) { return Vec{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]}; }
+    static __device__ inline Mma<float>::Acc mma(Vec a, Vec b, Mma<float>::Acc c) { return __builtin_amdgcn_mfma_f32_32x32x8f16(a, b, c, 0, 0, 0); }
+};
+
+template <typename S>
+__global__ void widen_kernel(const S* __restrict__ src, float* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::widen(src[i]);
+}
+template <typename S>
+__global__ void narrow_kernel(const float* __restrict__ src, S* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::narrow(src[i]);
+}
+
 
 // ---------------------------------------------------------------------------------------------
 // Weight re-layout into the workspace (tiny: the whole weight is at most a few MB).
@@ -61,6 +123,32 @@ __host__ __device__ inline int chunk_candidate(int cpg, int Cg, int y) {     // 
     if (big % seg) return y;
     const int cps = (seg + CCH - 1) / CCH;
     return y / cps * seg + y % cps * CCH;
+}
+
+// Operands of the grad-column GEMM of the fused backward kernel.  S = T: one value per lane and
+// reduction step, v_mfma_f32_32x32x2_f32 / v_mfma_f64_16x16x4_f64 (KS = KL output channels per
+// step).  S = Bf16 / Fp16 (T = float): four values per lane and step -- the output channels
+// 8 * step + 4 * (lane / 32) + 0..3 -- for v_mfma_f32_32x32x8_bf16 / _f16, which accumulate in float
+// and leave the result in the registers of the float instruction (KS = 8 output channels per step).
+template <typename T, typename S> struct GcolGemm {
+    static constexpr int KS = Mma<T>::KL;
+    typedef T Op;
+    __device__ static inline typename Mma<T>::Acc mma(Op a, Op b, typename Mma<T>::Acc c) { return Mma<T>::mma(a, b, c); }
+};
+template <> struct GcolGemm<float, Bf16> {
+    static constexpr int KS = 8;
+    typedef Mma16<Bf16>::Vec Op;
+    __device__ static inline Mma<float>::Acc mma(Op a, Op b, Mma<float>::Acc c) { return Mma16<Bf16>::mma(a, b, c); }
+};
+template <> struct GcolGemm<float, Fp16> {
+    static constexpr int KS = 8;
+    typedef Mma16<Fp16>::Vec Op;
+    __device__ static inline Mma<float>::Acc mma(Op a, Op b, Mma<float>::Acc c) { return Mma16<Fp16>::mma(a, b, c); }
+};
+// reduction steps of a weight slab's pass: a multiple of the largest operand batch
+template <typename T, typename S> __host__ __device__ inline int gcol_slab_steps(int M) {
+    constexpr bool S16 = !std::is_same<S, T>::value;
+    return S16 ? ((M + 7) / 8 + 7) / 8 * 8 : ((M + Mma<T>::KL - 1) / Mma<T>::KL + 15) / 16 * 16;
 }
 
 // One block of 256 threads chooses the halo plan of the launches that follow (see PlanChoice).
@@ -132,10 +220,13 @@ __device__ inline void choose_plan(const PlanChoice& pc, const S* __restrict__ o
 // of a tap in one lane (fused_row_tap / fused_row_channel).
 // `bounds` (two floats, may be null) is cleared for the weight_bounds_kernel that follows.
 // With pc.sel set the launch has one block more, which chooses the halo plan from the offsets.
-template <typename T, int CCH, bool WIDE = false>
-__global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restrict__ Wp, float* __restrict__ bounds,
-                                   PlanChoice pc, const T* __restrict__ off, size_t n_off) {
+// S = Bf16 / Fp16: Wp[slab][pass][k][lane][r] = W[m = 8 * k + 4 * q + r][...], four values per lane and step.
+template <typename T, int CCH, bool WIDE = false, typename S = T>
+__global__ void pack_weight_kernel(Params P, const S* __restrict__ W, S* __restrict__ Wp, float* __restrict__ bounds,
+                                   PlanChoice pc, const S* __restrict__ off, size_t n_off) {
     using MM = Mma<T>;
+    constexpr bool S16 = !std::is_same<S, T>::value;
+    constexpr int PER = S16 ? 4 : 1;                    // values per lane and reduction step
     const unsigned pack_blocks = pc.sel ? gridDim.x - 1 : gridDim.x;
     if (blockIdx.x == pack_blocks) {
         choose_plan(pc, off, n_off);
@@ -144,8 +235,8 @@ __global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restr
     if (bounds && blockIdx.x == 0 && threadIdx.x < 2) bounds[threadIdx.x] = 0.f;
     constexpr int TN = MM::TN, KL = MM::KL, TP = TN / CCH;
     const int npass = (P.kV + TP - 1) / TP;
-    const int kst = ((P.M + KL - 1) / KL + 15) / 16 * 16;       // operand batches are 8 or 16 reduction steps
-    const size_t per_chunk = (size_t)npass * kst * 64;
+    const int kst = gcol_slab_steps<T, S>(P.M);                 // operand batches are 8 or 16 (16-bit: 4 or 8) reduction steps
+    const size_t per_chunk = (size_t)npass * kst * 64 * PER;
     const size_t total = (size_t)chunk_candidates<CCH>(P.cpg, P.Cg, P.C_in) * per_chunk;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)pack_blocks * blockDim.x) {
         const int c0 = chunk_candidate<CCH>(P.cpg, P.Cg, (int)(i / per_chunk));      // candidate first channel of a chunk
@@ -153,11 +244,12 @@ __global__ void pack_weight_kernel(Params P, const T* __restrict__ W, T* __restr
         if ((c0 - seg_b) % CCH) continue;
         const int seg_e = min((c0 / P.cpg + 1) * P.cpg, (c0 / P.Cg + 1) * P.Cg);
         const size_t r = i % per_chunk;
-        const int lane = (int)(r % 64), k = (int)((r / 64) % kst), pass = (int)(r / 64 / kst);
+        const int sub = (int)(r % PER);
+        const int lane = (int)((r / PER) % 64), k = (int)((r / PER / 64) % kst), pass = (int)(r / PER / 64 / kst);
         const int q = lane / TN, j = lane % TN;
         const int jt = WIDE ? 2 * (j / 16) + (j / 4) % 2 : j / CCH, jc = WIDE ? 4 * ((j / 8) % 2) + j % 4 : j % CCH;
-        const int m = k * KL + q, tap = pass * TP + jt, c = c0 + jc, g = c0 / P.Cg;
-        T v = 0;
+        const int m = S16 ? k * 8 + q * 4 + sub : k * KL + q, tap = pass * TP + jt, c = c0 + jc, g = c0 / P.Cg;
+        S v = S();
         if (m < P.M && tap < P.kV && c < seg_e) v = W[(((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)) * P.kV + tap];
         Wp[(size_t)chunk_slot<CCH>(P.cpg, P.Cg, c0) * per_chunk + r] = v;
     }
@@ -341,8 +433,8 @@ __device__ inline void halo_table(const Params& P, const HaloPlan& H, const Tile
 // padded halo rows than the reads gain.)
 template <typename T, int CCH>
 __host__ __device__ inline constexpr int swizzle_groups() { return (sizeof(T) == 4 && CCH == 8) ? CCH / 4 : 1; }
-template <typename T, int CCH, int WGS>
-__device__ inline void halo_stage_interleaved(const Params& P, const HaloPlan& H, const T* __restrict__ chan0, int nch,
+template <typename T, int CCH, int WGS, typename S = T>
+__device__ inline void halo_stage_interleaved(const Params& P, const HaloPlan& H, const S* __restrict__ chan0, int nch,
                                               const unsigned* __restrict__ sTab, T* __restrict__ sIn, int* __restrict__ nonfinite) {
     constexpr int GPV = swizzle_groups<T, CCH>();
     bool bad = false;                  // a NaN or an infinity among the staged values
@@ -351,7 +443,7 @@ __device__ inline void halo_stage_interleaved(const Params& P, const HaloPlan& H
         const unsigned g = t == ~0u ? 0u : t;
         T val[CCH];
 #pragma unroll
-        for (int c = 0; c < CCH; ++c) val[c] = chan0[(size_t)min(c, nch - 1) * P.inV + g];   // CCH loads in flight
+        for (int c = 0; c < CCH; ++c) val[c] = Store<S>::ld(chan0[(size_t)min(c, nch - 1) * P.inV + g]);   // CCH loads in flight
         // cells outside the volume hold zero: samples in the rim read them with weight zero
 #pragma unroll
         for (int c = 0; c < CCH; ++c) bad = bad || !(fabs(val[c]) <= std::numeric_limits<T>::max());
@@ -478,35 +570,6 @@ __global__ __launch_bounds__(256) void global_path_prepare_kernel(Params P, cons
             if (c < (unsigned)P.C_in && v < P.inV) in_cl[base + (size_t)v * P.C_in + c] = tile[tx][i];
         }
     }
-}
-
-// 16-bit storage formats of the mixed-precision entry points: the tensors are widened to float
-// (exactly) before the float32 kernels run and the results are rounded once, to nearest even.
-struct Bf16 {       // bfloat16: the upper half of a float
-    unsigned short bits;
-    __device__ static inline float widen(Bf16 v) { return __uint_as_float((unsigned)v.bits << 16); }
-    __device__ static inline Bf16 narrow(float f) {
-        const unsigned u = __float_as_uint(f);
-        Bf16 r;
-        if ((u & 0x7fffffffu) > 0x7f800000u) r.bits = (unsigned short)((u >> 16) | 0x40u);      // NaN stays NaN
-        else r.bits = (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);                  // Inf and overflow to Inf included
-        return r;
-    }
-};
-struct Fp16 {       // IEEE binary16
-    _Float16 v;
-    __device__ static inline float widen(Fp16 x) { return (float)x.v; }
-    __device__ static inline Fp16 narrow(float f) { Fp16 r; r.v = (_Float16)f; return r; }
-};
-__device__ inline float offset_value(Bf16 v) { return Bf16::widen(v); }
-__device__ inline float offset_value(Fp16 v) { return Fp16::widen(v); }
-template <typename S>
-__global__ void widen_kernel(const S* __restrict__ src, float* __restrict__ dst, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::widen(src[i]);
-}
-template <typename S>
-__global__ void narrow_kernel(const float* __restrict__ src, S* __restrict__ dst, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = S::narrow(src[i]);
 }
 
 template <typename T>
@@ -840,7 +903,7 @@ __global__ __launch_bounds__(512) void weight_bounds_kernel(const T* __restrict_
         const T* p = w + (size_t)blockIdx.y * M * cols + col;
 #pragma unroll 8
         for (int r = sl; r < M; r += 8) {
-            const float v = (float)p[(size_t)r * cols];
+            const float v = offset_value(p[(size_t)r * cols]);
             ss += v * v;
             am = max(am, __float_as_uint(fabsf(v)));
         }
@@ -902,13 +965,16 @@ __global__ __launch_bounds__(512) void weight_bounds_kernel(const T* __restrict_
 // that (positions of the block x taps) of the largest possible one -- all that a cell can receive
 // -- still fit 31 bits; the host allows it only while that leaves enough bits below that term.
 // wmax[1] then holds the largest column norm of the weight (colnorm_max_kernel).
+// S: storage format of input, offset, weight and grad_output (Bf16 / Fp16 with T = float: the grad-column
+// GEMM then runs on the 16-bit matrix instructions, see GcolGemm; requires BREG and PACKW); the
+// gradients are written as T.
 template <typename T, int ND, int CCH, bool COORD, bool BREG, int HS, int NW, bool PACKW = false, bool PAIR = false, int BS = 1,
-          int HE1 = 0, int HE2 = 0>
+          int HE1 = 0, int HE2 = 0, typename S = T>
 __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
-                                                                  const T* __restrict__ in,
-                                                                  const T* __restrict__ off,
-                                                                  const T* __restrict__ Wt,
-                                                                  const T* __restrict__ gout,
+                                                                  const S* __restrict__ in,
+                                                                  const S* __restrict__ off,
+                                                                  const S* __restrict__ Wt,
+                                                                  const S* __restrict__ gout,
                                                                   const float* __restrict__ wmax,
                                                                   T* __restrict__ gin, T* __restrict__ goff, int csplit,
                                                                   unsigned whole, int goff_atomic) {
@@ -917,6 +983,11 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     using MM = Mma<T>;
     using Cell = typename LdsCell<T>::type;
     constexpr int TN = MM::TN, KL = MM::KL, NC = 1 << ND, NACC = MM::NACC;
+    constexpr bool S16 = !std::is_same<S, T>::value;
+    using GG = GcolGemm<T, S>;
+    using Op = typename GG::Op;                         // what a lane supplies to one reduction step
+    constexpr int KS = GG::KS;                          // output channels per reduction step
+    static_assert(!S16 || (BREG && PACKW && sizeof(T) == 4), "16-bit operands: packed weights, grad_output in registers");
     constexpr int TP = TN / CCH;                        // taps per MFMA pass
     // WIDE (paired cells, 8-channel chunks): the weight rows are ordered such that a lane receives
     // all eight channels of a tap -- lane group q the taps q and 2 + q of a pass -- instead of four
@@ -985,7 +1056,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     for (int a = 0; a < ND; ++a) ibf[a] = (T)ib[a];
 
     const int c_lo = dg * P.cpg, c_hi = c_lo + P.cpg;
-    const T* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
+    const S* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
     T* goff_dg = goff + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
     bool first_chunk = true;                        // grad_offset without atomics: the first channel chunk stores, later ones add
     int chunk_no = 0;
@@ -996,10 +1067,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
     for (int g = c_lo / P.Cg; g <= (c_hi - 1) / P.Cg; ++g) {
         const int rb = max(c_lo, g * P.Cg), re = min(c_hi, (g + 1) * P.Cg);
         // wave-uniform base (scalar registers) + 32-bit lane offset of the B operand grad_output[m][pos]
-        constexpr int AB = (WIDE || CCH == 16) ? 16 : 8;      // reduction steps per operand batch (NS * AB = 32 ride on a pass)
-        const T* gbase = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV;
+        constexpr int AB = ((WIDE || CCH == 16) ? 16 : 8) / (S16 ? 2 : 1);      // reduction steps per operand batch (NS * AB ride on a pass: 64 output channels, 16-bit 128)
+        const S* gbase = gout + ((size_t)n * P.C_out + (size_t)g * P.M) * P.outV;
         const unsigned b_off = (unsigned)q * P.outV + pos;
-        const size_t gstep = (size_t)KL * P.outV;
+        const size_t gstep = (size_t)KS * P.outV;
         // Reduction step k of this lane reads grad_output[k * KL + q][pos]: the row base advances in
         // scalar registers, clamped at the last real step (the further steps of a batch meet zero
         // weight rows and re-read that step; a lane whose row of the last step lies past M reads
@@ -1008,13 +1079,41 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
         // address arithmetic per lane.  Lanes outside the volume read a clamped position (their
         // columns are never used).  No load is masked: a masked load becomes a conditional one,
         // issued alone with a full wait behind it.
-        const int klast = (P.M + KL - 1) / KL - 1;
+        const int klast = (P.M + KS - 1) / KS - 1;
         const unsigned b_byte = b_off * (unsigned)sizeof(T);
         const unsigned b_byte_last = (klast * KL + q < P.M ? b_off : pos) * (unsigned)sizeof(T);
-        T b_reg[BREG ? NS * AB * BS : 1];
+        Op b_reg[BREG ? NS * AB * BS : 1];
         float sabs = 0.f;                           // sum_m |grad_output| of this lane's position (its q share); PAIR: of the squares
         float amax = 0.f;                           // PAIR: largest |grad_output| seen (squares of tiny values underflow)
-        if constexpr (BREG) {
+        if constexpr (S16) {
+            // four output channels per lane and step: rows 8 * k + 4 * q + r of grad_output at this lane's
+            // position; rows past M (last step only: zero weights there) re-read row M - 1
+            int kl = klast;
+            asm volatile("" : "+s"(kl));
+            unsigned row_off[4], row_off_last[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                row_off[r] = ((unsigned)(4 * q + r) * P.outV + pos) * (unsigned)sizeof(S);
+                const int rl = min(kl * 8 + 4 * q + r, P.M - 1) - kl * 8;
+                row_off_last[r] = ((unsigned)rl * P.outV + pos) * (unsigned)sizeof(S);
+            }
+            const char* gk = reinterpret_cast<const char*>(gbase);
+#pragma unroll
+            for (int k = 0; k < NS * AB * BS; ++k) {
+                float g4[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    g4[r] = Store<S>::ld(*reinterpret_cast<const S*>(gk + (k >= kl ? row_off_last[r] : row_off[r])));
+                gk += k < kl ? gstep * sizeof(S) : (size_t)0;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool counts = valid && k <= kl && k * 8 + 4 * q + r < P.M;
+                    sabs += counts ? (PAIR ? g4[r] * g4[r] : fabsf(g4[r])) : 0.f;
+                    if constexpr (PAIR) amax = counts ? fmaxf(amax, fabsf(g4[r])) : amax;
+                }
+                b_reg[k] = Mma16<S>::pack(g4);          // (exact: the values are 16-bit already)
+            }
+        } else if constexpr (BREG) {
             // held unmasked (rows past M meet zero weight rows, columns outside the volume are never
             // used): a masked load becomes a conditional one, issued alone with a full wait behind it
             // (the last step passes through an empty asm: the per-step selects derived from it are
@@ -1120,7 +1219,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             __syncthreads();                        // the previous chunk's flush is done
             for (int c = 0; c < (PAIR ? (nch + 1) / 2 : nch); ++c)
                 for (int v = threadIdx.x; v < H.hvol; v += WGS) sG[c * hs + v] = 0;      // all-zero bits in either cell type
-            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS>(P, H, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn, &sNonFinite);
+            if constexpr (COORD) halo_stage_interleaved<T, CCH, WGS, S>(P, H, in + ((size_t)n * P.C_in + cc0) * P.inV, nch, sTab, sIn, &sNonFinite);
             __syncthreads();
             // Non-finite input values in this halo: the branch-free sampler reads the cell next to a
             // collapsed corner with weight 0, and 0 * inf would be NaN where the reference never
@@ -1135,22 +1234,24 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             // the matrix pipe works behind the vector work of the scatter instead of before it.
             // Operands arrive in batches of AB reduction steps, loaded one tap slot ahead of use.
             constexpr int MPR = AB / RPS;                              // MFMAs per accumulator register walked
-            const int ksteps = (P.M + KL - 1) / KL;
+            const int ksteps = (P.M + KS - 1) / KS;
+            // (weights are addressed in operands: one value, or with 16-bit storage four values, per lane and step)
+            const Op* Wo = reinterpret_cast<const Op*>(Wt);
             const size_t wstep = PACKW ? (size_t)64 : (size_t)KL * P.Cgp;
-            const size_t wpass = PACKW ? (size_t)((ksteps + 15) / 16 * 16) * 64 : (size_t)TP * P.Mp * P.Cgp;   // weights of one pass
-            const T* wchunk = PACKW ? Wt + (size_t)chunk_slot<CCH>(P.cpg, P.Cg, cc0) * ((P.kV + TP - 1) / TP) * wpass
-                                    : Wt + ((size_t)g * P.kV * P.Mp) * P.Cgp + (cc0 - g * P.Cg);      // uniform; lanes add a_off
+            const size_t wpass = PACKW ? (size_t)gcol_slab_steps<T, S>(P.M) * 64 : (size_t)TP * P.Mp * P.Cgp;   // weights of one pass
+            const Op* wchunk = PACKW ? Wo + (size_t)chunk_slot<CCH>(P.cpg, P.Cg, cc0) * ((P.kV + TP - 1) / TP) * wpass
+                                     : Wo + ((size_t)g * P.kV * P.Mp) * P.Cgp + (cc0 - g * P.Cg);      // uniform; lanes add a_off
             // (k0 passes through an empty asm: what is derived from it is then computed where it is
             // used instead of being hoisted out of the loops into hundreds of long-lived registers)
-            auto load_batch = [&](T* a_nx, T* b_nx, const T* wp, int k0) {      // rows past M are zero padding
+            auto load_batch = [&](Op* a_nx, Op* b_nx, const Op* wp, int k0) {      // rows past M are zero padding
                 asm volatile("" : "+s"(k0));
-                const T* wb = wp + (size_t)k0 * wstep;                 // one 64-bit product per batch; the row offsets below are loop invariants
+                const Op* wb = wp + (size_t)k0 * wstep;                // one 64-bit product per batch; the row offsets below are loop invariants
                 const char* gk = reinterpret_cast<const char*>(gbase + (size_t)min(k0, klast) * gstep);
 #pragma unroll
                 for (int k = 0; k < AB; ++k) {
                     a_nx[k] = (wb + (unsigned)k * (unsigned)wstep)[a_off];
                     if constexpr (!BREG) {
-                        b_nx[k] = *reinterpret_cast<const T*>(gk + (k0 + k >= klast ? b_byte_last : b_byte));
+                        b_nx[k] = *reinterpret_cast<const Op*>(gk + (k0 + k >= klast ? b_byte_last : b_byte));
                         gk += k0 + k < klast ? gstep * sizeof(T) : (size_t)0;
                     }
                 }
@@ -1160,8 +1261,8 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
             // (two operand sets that swap roles from batch to batch, two batches per loop trip: copying
             // "next" into "current" costs 2 * AB register moves per batch whenever the register
             // allocator cannot merge the sets, on the same issue port as the MFMAs)
-            auto gemm_tail = [&](typename MM::Acc& dd, const T* wp, int k_begin) {
-                T a_s[2][AB], b_s[2][AB];
+            auto gemm_tail = [&](typename MM::Acc& dd, const Op* wp, int k_begin) {
+                Op a_s[2][AB], b_s[2][AB];
                 load_batch(a_s[0], b_s[0], wp, k_begin);
                 int k0 = k_begin;
                 if (PACKW && ksteps - k_begin >= 96) {
@@ -1176,14 +1277,14 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     // grad_output rows: two scalar adds per load instead of a dozen scalar instructions,
                     // which a wavefront has to issue between two MFMAs.
                     const int kfast_end = P.M % KL == 0 ? klast + 1 : klast;      // steps [0, kfast_end) load without a clamp
-                    auto load_fast = [&](T* a_nx, T* b_nx, int k0f) {
+                    auto load_fast = [&](Op* a_nx, Op* b_nx, int k0f) {
                         asm volatile("" : "+s"(k0f));
-                        const T* wb = wp + (size_t)k0f * wstep;
+                        const Op* wb = wp + (size_t)k0f * wstep;
                         const char* gk = reinterpret_cast<const char*>(gbase + (size_t)k0f * gstep);
 #pragma unroll
                         for (int k = 0; k < AB; ++k) {
                             a_nx[k] = (wb + (unsigned)k * (unsigned)wstep)[a_off];
-                            b_nx[k] = *reinterpret_cast<const T*>(gk + b_byte);
+                            b_nx[k] = *reinterpret_cast<const Op*>(gk + b_byte);
                             gk += gstep * sizeof(T);
                         }
                     };
@@ -1200,27 +1301,27 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         for (; k0 + 3 * AB <= kfast_end; k0 += 2 * AB) {
                             load_fast(a_s[1], b_s[1], k0 + AB);
 #pragma unroll
-                            for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                            for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[0][k], b_s[0][k], dd);
                             deal();
                             load_fast(a_s[0], b_s[0], k0 + 2 * AB);
 #pragma unroll
-                            for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[1][k], b_s[1][k], dd);
+                            for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[1][k], b_s[1][k], dd);
                             deal();
                         }
                     }
                     for (; k0 + AB < ksteps; k0 += 2 * AB) {
                         load_batch(a_s[1], b_s[1], wp, min(k0 + AB, k_last));
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                        for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[0][k], b_s[0][k], dd);
                         deal();
                         load_batch(a_s[0], b_s[0], wp, min(k0 + 2 * AB, k_last));
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[1][k], b_s[1][k], dd);
+                        for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[1][k], b_s[1][k], dd);
                         deal();
                     }
                     if (k0 < ksteps) {
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                        for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[0][k], b_s[0][k], dd);
                     }
                     return;
                 }
@@ -1228,30 +1329,30 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     load_batch(a_s[1], b_s[1], wp, k0 + AB);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                    for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[0][k], b_s[0][k], dd);
                     __builtin_amdgcn_sched_barrier(0);
                     if (k0 + 2 * AB < ksteps) load_batch(a_s[0], b_s[0], wp, k0 + 2 * AB);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[1][k], b_s[1][k], dd);
+                    for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[1][k], b_s[1][k], dd);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (k0 < ksteps) {
 #pragma unroll
-                    for (int k = 0; k < AB; ++k) dd = MM::mma(a_s[0][k], b_s[0][k], dd);
+                    for (int k = 0; k < AB; ++k) dd = GG::mma(a_s[0][k], b_s[0][k], dd);
                 }
             };
             // register-resident operand: the batches of a pass past those that ride on the tap slots
-            auto gemm_tail_reg = [&](typename MM::Acc& dd, const T* wp) {
+            auto gemm_tail_reg = [&](typename MM::Acc& dd, const Op* wp) {
                 if constexpr (BREG && BS > 1) {
-                    T a_x[2][AB];
+                    Op a_x[2][AB];
                     if (NS * AB < ksteps) load_batch(a_x[0], nullptr, wp, NS * AB);
 #pragma unroll
                     for (int kb = NS; kb < NS * BS; ++kb) {
                         if (kb * AB < ksteps) {
                             if ((kb + 1) * AB < ksteps && kb + 1 < NS * BS) load_batch(a_x[(kb + 1 - NS) & 1], nullptr, wp, (kb + 1) * AB);
 #pragma unroll
-                            for (int k = 0; k < AB; ++k) dd = MM::mma(a_x[(kb - NS) & 1][k], b_reg[kb * AB + k], dd);
+                            for (int k = 0; k < AB; ++k) dd = GG::mma(a_x[(kb - NS) & 1][k], b_reg[kb * AB + k], dd);
                         }
                     }
                 }
@@ -1261,10 +1362,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                 for (int ts = 0; ts < NS; ++ts) {
                     if (ts * AB < ksteps) {
-                        T a_cu[AB];
+                        Op a_cu[AB];
                         load_batch(a_cu, nullptr, wchunk, ts * AB);
 #pragma unroll
-                        for (int k = 0; k < AB; ++k) d_next = MM::mma(a_cu[k], b_reg[ts * AB + k], d_next);
+                        for (int k = 0; k < AB; ++k) d_next = GG::mma(a_cu[k], b_reg[ts * AB + k], d_next);
                     }
                 }
                 gemm_tail_reg(d_next, wchunk);
@@ -1303,9 +1404,9 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 const int dq = row_tap(ts * RPS, q) - row_tap(ts * RPS, 0);
                 const int dqc = tu + dq < P.kV ? dq : 0;
                 const unsigned lo = (unsigned)dqc * ND * P.outV + pos;
-                const T* ob = off_dg + (size_t)tu * ND * P.outV;
+                const S* ob = off_dg + (size_t)tu * ND * P.outV;
 #pragma unroll
-                for (int a = 0; a < ND; ++a) o_nx[a] = (ob + (size_t)a * P.outV)[lo];
+                for (int a = 0; a < ND; ++a) o_nx[a] = Store<S>::ld((ob + (size_t)a * P.outV)[lo]);
                 if constexpr (RMW) {
                     if (rmw_prev) {
                         const T* gb = goff_dg + (size_t)tu * ND * P.outV;
@@ -1362,7 +1463,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                 const bool more = tap0 + TP < P.kV;                    // a pass follows: its MFMAs ride along
                 int kz = 0;                                            // an opaque zero, for the same reason
                 asm volatile("" : "+s"(kz));
-                const T* wnext = wchunk + (size_t)(tap0 / TP + 1) * wpass;
+                const Op* wnext = wchunk + (size_t)(tap0 / TP + 1) * wpass;
                 if constexpr (!BREG) { if (more && ksteps > NS * AB) gemm_tail(d_next, wnext, NS * AB); }
                 else { if (more) gemm_tail_reg(d_next, wnext); }
 #pragma unroll
@@ -1370,7 +1471,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                     // slots past the last tap (only in the last pass, which feeds no further MFMAs)
                     if (tap0 + row_tap(ts * RPS, 0) >= P.kV) continue;
                     const int tap = tap0 + row_tap(ts * RPS, q);
-                    T a_cu[AB], b_cu[AB];
+                    Op a_cu[AB], b_cu[AB];
                     const T* ofs = o_buf[ts & 1];
                     const T* kdf = kd_buf[ts & 1];
                     const bool do_mma = more && ts * AB < ksteps;      // uniform
@@ -1481,7 +1582,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                         if (do_mma) {
 #pragma unroll
                             for (int k = h * (AB / RH); k < (h + 1) * (AB / RH); ++k)
-                                d_next = MM::mma(a_cu[k], BREG ? b_reg[ts * AB + k] : b_cu[k], d_next);
+                                d_next = GG::mma(a_cu[k], BREG ? b_reg[ts * AB + k] : b_cu[k], d_next);
                         }
                         if constexpr (COORD) {
 #pragma unroll
@@ -1584,10 +1685,10 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
 #pragma unroll
                                 for (int i = 0; i < NC; ++i) atomic_add(gc + t.idx[i], fcw[i] * g1);
                                 if constexpr (COORD) {
-                                    const T* ic = in + chan;
+                                    const S* ic = in + chan;
                                     T v[NC];
 #pragma unroll
-                                    for (int i = 0; i < NC; ++i) v[i] = g1 * ic[t.idx[i]];
+                                    for (int i = 0; i < NC; ++i) v[i] = g1 * Store<S>::ld(ic[t.idx[i]]);
                                     if constexpr (ND == 3) {
                                         const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
                                         const T c00 = v[0] * gw + v[1] * fw, c01 = v[2] * gw + v[3] * fw;
