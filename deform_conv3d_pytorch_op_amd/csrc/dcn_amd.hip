@@ -1317,6 +1317,66 @@ int backward_input_offset16(const Geometry& g, const S* in, const S* w, const S*
     if (int rc = narrow(fgin, gin, z.in, s)) return rc;
     return narrow(fgoff, goff, z.off, s);
 }
+// backward_weight on the 16-bit tensors themselves (backward_weight16_kernel): channels-last copies of
+// the input and of grad_output in their storage format, the offsets as they are, float partial tiles.
+// Declines (nothing launched) where the kernel's 4-byte loads of channel pairs would not be aligned
+// (an odd number of input channels, or segments -- intersections of convolution groups and deformable
+// groups -- that start at odd channels) or the workspace is too small for it.
+template <typename S, int ND>
+int backward_weight_native16(const Params& Pin, const S* in, const S* off, const S* gout, float* fgw, void* ws, size_t ws_bytes,
+                             hipStream_t s, bool* declined) {
+    Params P = Pin;
+    const int TN = Mma<float>::TN, CT = 2 * TN;
+    *declined = true;
+    if (P.C_in % 2 || P.cpg % 2 || P.Cg % 2) return DCN_OK;
+    if ((unsigned long long)P.inV * P.C_in * sizeof(S) >= (1ull << 32) || (unsigned long long)P.outV * P.C_out >= (1ull << 32)) return DCN_OK;
+    if (2 * (long long)P.N > 65535) return DCN_OK;
+    const int mtiles = (P.M + TN - 1) / TN;
+    const int MT = mtiles >= 2 ? 2 : 1;             // (four row tiles would take 128 accumulator registers beside the two channel tiles)
+    P.mchunks = (mtiles + MT - 1) / MT;
+    P.nctiles = 0;
+    for (int gg = 0; gg < P.G; ++gg) {
+        const int cg0 = gg * P.Cg, cg1 = cg0 + P.Cg;
+        for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+            const int cb = cg0 > dg * P.cpg ? cg0 : dg * P.cpg, ce = cg1 < (dg + 1) * P.cpg ? cg1 : (dg + 1) * P.cpg;
+            P.nctiles += (ce - cb + CT - 1) / CT;
+        }
+    }
+    // position splits: about 2560 workgroups, as in the float kernel's plan
+    const long long slabs = (long long)P.N * ((P.outV + TN - 1) / TN), other = (long long)P.kV * P.nctiles * P.mchunks;
+    long long split = (2560 + other - 1) / other;
+    const long long max_split = (slabs + WAVES - 1) / WAVES;
+    if (split > max_split) split = max_split;
+    if (split > 256) split = 256;
+    if (split < 1) split = 1;
+    P.nsplit = (int)split;
+    if ((long long)P.nsplit * other > 0x7fffffffLL) return DCN_OK;
+    const size_t ibytes = align256((size_t)P.N * P.C_in * P.inV * sizeof(S));
+    const size_t obytes = align256((size_t)P.N * P.C_out * P.outV * sizeof(S));
+    const size_t pbytes = align256((size_t)P.nsplit * P.kV * P.C_out * P.Cg * sizeof(float));
+    if (!ws || ws_bytes < ibytes + obytes + pbytes) return DCN_OK;
+    *declined = false;
+    S* in_cl = static_cast<S*>(ws);
+    S* gout_cl = reinterpret_cast<S*>(static_cast<char*>(ws) + ibytes);
+    float* partial = reinterpret_cast<float*>(static_cast<char*>(ws) + ibytes + obytes);
+    {
+        const unsigned vmax = P.inV > P.outV ? P.inV : P.outV;
+        const int cmax = P.C_in > P.C_out ? P.C_in : P.C_out;
+        hipLaunchKernelGGL(to_channels_last_pair_kernel<S>, dim3((vmax + 31) / 32, (unsigned)(cmax + 31) / 32, 2u * (unsigned)P.N), dim3(32, 8), 0, s,
+                           in, in_cl, P.C_in, P.inV, gout, gout_cl, P.C_out, P.outV, P.N);
+        if (int rc = check_launch("to_channels_last_pair_kernel")) return rc;
+    }
+    const size_t lds = (size_t)WAVES * TN * (TN + 1) * sizeof(float);
+    const dim3 grid((unsigned)(P.nsplit * other));
+    if (MT == 2) hipLaunchKernelGGL((backward_weight16_kernel<ND, 2, S>), grid, dim3(WG), lds, s, P, (const S*)in_cl, off, (const S*)gout_cl, partial);
+    else hipLaunchKernelGGL((backward_weight16_kernel<ND, 1, S>), grid, dim3(WG), lds, s, P, (const S*)in_cl, off, (const S*)gout_cl, partial);
+    if (int rc = check_launch("backward_weight16_kernel")) return rc;
+    const size_t rows_x_cg = (size_t)P.C_out * P.Cg, total = rows_x_cg * P.kV;
+    const unsigned rb = (unsigned)((total + 63) / 64 > 8192 ? 8192 : (total + 63) / 64);
+    hipLaunchKernelGGL(reduce_weight_partials_kernel<float>, dim3(rb), dim3(256), 0, s, (const float*)partial, fgw, P.nsplit, P.kV, rows_x_cg);
+    return check_launch("reduce_weight_partials_kernel");
+}
+
 template <typename S, int ND>
 int backward_weight16(const Geometry& g, const S* in, const S* off, const S* gout, S* gw, void* ws, size_t ws_bytes, hipStream_t s) {
     Params P;
@@ -1327,11 +1387,16 @@ int backward_weight16(const Geometry& g, const S* in, const S* off, const S* gou
     Carver c{static_cast<char*>(ws), ws ? ws_bytes : 0};
     float *fin = c.take(z.in), *foff = c.take(z.off), *fgout = c.take(z.out), *fgw = c.take(z.w);
     if (!fin || !foff || !fgout || !fgw) return fail(DCN_E_WORKSPACE, "workspace too small");
-    if (int rc = widen(in, fin, z.in, s)) return rc;
-    if (int rc = widen(off, foff, z.off, s)) return rc;
-    if (int rc = widen(gout, fgout, z.out, s)) return rc;
     if (int rc = widen(gw, fgw, z.w, s)) return rc;               // grad_weight is accumulated into
-    if (int rc = backward_weight<float, ND>(g, fin, foff, fgout, fgw, c.p, c.left, s)) return rc;
+    bool declined = true;
+    if (native16())
+        if (int rc = backward_weight_native16<S, ND>(P, in, off, gout, fgw, c.p, c.left, s, &declined)) return rc;
+    if (declined) {
+        if (int rc = widen(in, fin, z.in, s)) return rc;
+        if (int rc = widen(off, foff, z.off, s)) return rc;
+        if (int rc = widen(gout, fgout, z.out, s)) return rc;
+        if (int rc = backward_weight<float, ND>(g, fin, foff, fgout, fgw, c.p, c.left, s)) return rc;
+    }
     return narrow(fgw, gw, z.w, s);
 }
 

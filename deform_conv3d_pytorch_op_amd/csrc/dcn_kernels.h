@@ -1957,6 +1957,218 @@ __global__ __launch_bounds__(WG) void backward_weight_kernel(Params P, const T* 
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Backward to weight with 16-bit storage (S = Bf16 / Fp16, float arithmetic): the same
+// decomposition as backward_weight_kernel -- a workgroup keeps one (tap, channel tile, m chunk),
+// its wavefronts stride over slabs of TN positions, one partial tile per split -- on the 16-bit
+// matrix instructions v_mfma_f32_32x32x8_bf16 / _f16 (float accumulation).  One instruction reduces
+// over 8 positions: lane (j, q) supplies the positions 8 * step + 4 * q + 0..3 of its row / column.
+//  * B operand (sampled columns): the input is held channels-last in its storage format and a lane
+//    fetches TWO neighbouring channels of a corner with one 4-byte load, so a channel tile is 64
+//    channels wide (columns j of two accumulator tiles: channels first + 2 j and first + 2 j + 1) and
+//    a sample costs half the load instructions of the float kernel; interpolation in float, the
+//    sampled values rounded to the storage format for the matrix instruction (as the forward pass
+//    does).  The host calls this kernel only for an even number of input channels with even
+//    segment starts (4-byte alignment of the channel pairs).
+//  * A operand: grad_output channels-last in its storage format ([n][position][output channel]): the
+//    lanes of a load read consecutive output channels of one position (in grad_output's own layout
+//    every lane of a load would touch a cache line of its own).
+// dynamic LDS = WAVES * TN * (TN + 1) * 4 bytes, as in the float kernel.
+template <int ND, int MT, typename S>
+__global__ __launch_bounds__(WG) void backward_weight16_kernel(Params P, const S* __restrict__ in_cl, const S* __restrict__ off,
+                                                               const S* __restrict__ gout_cl, float* __restrict__ partial) {
+    typedef float T;
+    using MM = Mma<float>;
+    constexpr int TN = MM::TN, NC = 1 << ND, CT = 2 * TN;          // CT channels per tile
+    __shared__ __align__(16) unsigned sIdx[WAVES][TN][NC];   // byte offset of each corner's channel 0 inside the sample, 0 when the sample is dead
+    __shared__ __align__(16) T sCw[WAVES][TN][NC];           // interpolation weight of each corner, 0 when the sample is dead
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sAcc = reinterpret_cast<T*>(smem_raw);                // [WAVES][TN][TN + 1]
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane % TN, q = lane / TN;
+
+    const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int tap = wg % (unsigned)P.kV;
+    const int split = (wg / (unsigned)P.kV) % (unsigned)P.nsplit;
+    const unsigned zz = (wg / (unsigned)P.kV) / (unsigned)P.nsplit;
+    const int mchunk = zz % P.mchunks;
+    int z = zz / P.mchunks;
+    int g = 0, dg = 0, c0 = 0, ce = 0;
+    bool found = false;
+    for (g = 0; g < P.G && !found; ++g) {
+        const int cg0 = g * P.Cg, cg1 = cg0 + P.Cg;
+        for (dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
+            const int cb = max(cg0, dg * P.cpg);
+            ce = min(cg1, (dg + 1) * P.cpg);
+            const int nt = (ce - cb + CT - 1) / CT;
+            if (z < nt) { c0 = cb + z * CT; found = true; break; }
+            z -= nt;
+        }
+        if (found) break;
+    }
+    if (!found) return;     // uniform for the workgroup
+
+    int kk[ND], kd[ND];
+    decode_tap<ND>(P, tap, kk);
+#pragma unroll
+    for (int a = 0; a < ND; ++a) kd[a] = kk[a] * P.dil[slot<ND>(a)];
+
+    typename MM::Acc acc[2][MT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = acc_zero<T>();
+
+    const int m_base = mchunk * MT * TN;
+    // this lane's channel pair (clamped to the last whole pair of the tensor: dead lanes still load legally)
+    const unsigned cjB = (unsigned)min(c0 + 2 * j, P.C_in - 2) * (unsigned)sizeof(S);
+    const unsigned cinB = (unsigned)P.C_in * (unsigned)sizeof(S);
+    unsigned mrow[MT];                              // this lane's output channel (clamped: rows past M are not stored)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) mrow[mt] = (unsigned)(g * P.M + min(m_base + mt * TN + j, P.M - 1));
+
+    const int slabs_per_sample = (P.outV + TN - 1) / TN;
+    const int nslabs = P.N * slabs_per_sample;
+    for (int slab = split * WAVES + wave; slab < nslabs; slab += P.nsplit * WAVES) {
+        const int n = slab / slabs_per_sample;
+        const unsigned p0 = (unsigned)(slab % slabs_per_sample) * TN;
+        const unsigned pos = p0 + j;
+        const bool valid = pos < P.outV;
+        const unsigned posc = valid ? pos : P.outV - 1;
+        int o[ND], ib[ND];
+        decode_pos<ND>(P, posc, o);
+#pragma unroll
+        for (int a = 0; a < ND; ++a) ib[a] = o[a] * P.stride[slot<ND>(a)] - P.pad[slot<ND>(a)];
+        TapGeo<T, ND> t;
+        {
+            const S* op = off + (((size_t)n * P.DG + dg) * P.kV + tap) * ND * P.outV;
+            T offv[ND];
+#pragma unroll
+            for (int a = 0; a < ND; ++a) offv[a] = Store<S>::ld(op[(size_t)a * P.outV + posc]);
+            tap_setup_noidx<T, ND>(P, offv, ib, kd, t);
+        }
+        const bool live = valid && t.inside;
+
+        // LDS operations of one wavefront execute in order; the fences only pin the compiler
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (q == 0) {
+            T cw[NC];                              // multiplied in the reference's order (w_l * w_h * w_w)
+            if constexpr (ND == 3) {
+                const T fl = t.f[0], gl = (T)1 - fl, fh = t.f[1], gh = (T)1 - fh, fw = t.f[2], gw = (T)1 - fw;
+                cw[0] = gl * gh * gw; cw[1] = gl * gh * fw; cw[2] = gl * fh * gw; cw[3] = gl * fh * fw;
+                cw[4] = fl * gh * gw; cw[5] = fl * gh * fw; cw[6] = fl * fh * gw; cw[7] = fl * fh * fw;
+            } else {
+                const T fh = t.f[0], gh = (T)1 - fh, fw = t.f[1], gw = (T)1 - fw;
+                cw[0] = gh * gw; cw[1] = gh * fw; cw[2] = fh * gw; cw[3] = fh * fw;
+            }
+            unsigned cb[NC];
+            tap_corner_offsets<T, ND>(P, t, live, cinB, cb);
+#pragma unroll
+            for (int i = 0; i < NC; ++i) sIdx[wave][j][i] = cb[i];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) sCw[wave][j][i] = live ? cw[i] : (T)0;      // a dead sample weighs nothing
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        const char* in_n = reinterpret_cast<const char*>(in_cl + (size_t)n * P.inV * P.C_in);        // scalar bases
+        const S* go_n = gout_cl + (size_t)n * P.C_out * P.outV;
+        constexpr int NK = TN / 8;                  // matrix instructions (reduction steps of 8 positions) per slab
+        // Software pipeline over the TN / 2 (position, lane group) units of the slab with the corner
+        // pairs of four units in flight (a ring of four register sets: unit u is interpolated from set
+        // u % 4, which then takes the loads of unit u + 4); every fourth unit completes a reduction
+        // step, whose grad_output rows were requested a step earlier.
+        constexpr int RING = 4;
+        unsigned cn[RING][NC];
+        typename Mma16<S>::Vec an[MT];
+        auto fetch_corners = [&](int u) {           // unit u: position 8 * (u / 4) + 4 * q + u % 4 of the slab
+            const int pp = (u / 4) * 8 + 4 * q + (u % 4);
+            unsigned ix[NC];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) ix[i] = sIdx[wave][pp][i];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) cn[u % RING][i] = *reinterpret_cast<const unsigned*>(in_n + (ix[i] + cjB));      // two channels
+        };
+        auto fetch_rows = [&](int ks) {             // A[row = m][k = position]: four consecutive positions, clamped at the end of the sample
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                S a4[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) a4[r] = go_n[min(p0 + (unsigned)(ks * 8 + 4 * q + r), P.outV - 1) * (unsigned)P.C_out + mrow[mt]];
+                an[mt] = __builtin_bit_cast(typename Mma16<S>::Vec, a4);
+            }
+        };
+        fetch_rows(0);
+#pragma unroll
+        for (int u = 0; u < RING; ++u) fetch_corners(u);
+        float ve[4], vo[4];                         // even / odd channel of the pair at the step's four positions
+#pragma unroll
+        for (int u = 0; u < NK * 4; ++u) {
+            unsigned cc[NC];
+            T wc[NC];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) cc[i] = cn[u % RING][i];
+            {
+                const int pp = (u / 4) * 8 + 4 * q + (u % 4);
+#pragma unroll
+                for (int i = 0; i < NC; ++i) wc[i] = sCw[wave][pp][i];
+            }
+            typename Mma16<S>::Vec ac[MT];
+            if (u % 4 == 3) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) ac[mt] = an[mt];
+                if (u / 4 + 1 < NK) fetch_rows(u / 4 + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            float se = 0.f, so = 0.f;
+#pragma unroll
+            for (int i = 0; i < NC; ++i) {
+                const unsigned short lb = (unsigned short)(cc[i] & 0xffffu), hb = (unsigned short)(cc[i] >> 16);
+                se += wc[i] * Store<S>::ld(__builtin_bit_cast(S, lb));
+                so += wc[i] * Store<S>::ld(__builtin_bit_cast(S, hb));
+            }
+            // (dead samples and positions past the end carry weight zero; an input value that is not
+            // finite there gives NaN, as 0 * inf does in the reference's GEMM on its zero column rows)
+            ve[u % 4] = se;
+            vo[u % 4] = so;
+            if (u + RING < NK * 4) fetch_corners(u + RING);       // into the set just consumed
+            if (u % 4 == 3) {
+                const typename Mma16<S>::Vec be = Mma16<S>::pack(ve), bo = Mma16<S>::pack(vo);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    acc[0][mt] = Mma16<S>::mma(ac[mt], be, acc[0][mt]);
+                    acc[1][mt] = Mma16<S>::mma(ac[mt], bo, acc[1][mt]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    constexpr int LDA = TN + 1;
+    T* pt = partial + ((size_t)split * P.kV + tap) * P.C_out * P.Cg;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            __syncthreads();                        // readers of the previous tile are done
+#pragma unroll
+            for (int r = 0; r < MM::NACC; ++r) sAcc[((size_t)wave * TN + MM::row(r, q)) * LDA + j] = acc[t2][mt][r];
+            __syncthreads();
+            for (int e = threadIdx.x; e < TN * TN; e += WG) {
+                const int mr = e / TN, cc = e % TN;
+                const int m = m_base + mt * TN + mr, c = c0 + 2 * cc + t2;
+                if (m < P.M && c < ce) {
+                    T sum = 0;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) sum += sAcc[((size_t)w * TN + mr) * LDA + cc];
+                    pt[((size_t)g * P.M + m) * P.Cg + (c - g * P.Cg)] = sum;
+                }
+            }
+        }
+}
+
 // grad_weight[g*M+m][cl][tap] += sum over splits of partial[split][tap][g*M+m][cl]
 // 256 threads = 64 consecutive elements x 4 lanes of splits: lane l adds the splits l, l + 4, ...
 // (loads of a lane independent of each other), then the four sums are added in the order of l, so

@@ -1,6 +1,8 @@
 """16-bit storage entry points (dcn*_bf16, dcn*_f16) through the package's Functions: every tensor is
-stored as bfloat16 / binary16.  Backward to weight: the tensors are widened exactly, the arithmetic is the
-float32 kernel's and each result is rounded once.  Backward to input and offset: the fused kernel reads the
+stored as bfloat16 / binary16.  Backward to weight: like the forward pass, the columns are sampled in float32
+from the 16-bit input, rounded to the storage format and multiplied with grad_output in 16-bit matrix
+instructions with float32 accumulation (layers with an odd number of input channels: widened and computed by
+the float32 kernel).  Backward to input and offset: the fused kernel reads the
 16-bit tensors, forms the grad columns with 16-bit matrix instructions (exact products, float32 sums) and
 each result is rounded once.  Forward: the columns are sampled in float32,
 rounded to the storage format and multiplied with the weights in 16-bit matrix instructions with
@@ -68,16 +70,16 @@ def test_16bit_storage_random_geometries_match_oracle(seed):
         _compare(make_case(*spec, dtype=dtype, seed=300 + seed), dtype, "random16_%d" % seed)
 
 
-def test_16bit_gradients_are_the_float32_gradients_rounded_once():
-    """backward_weight widens the tensors exactly, runs the float32 kernel and rounds once; backward_input_offset
-    reads the 16-bit tensors itself and multiplies them in 16-bit matrix instructions with float32 accumulation
-    -- the products of 16-bit values are exact in float32, so only the order of the sums differs from the float32
-    kernel -- and rounds once as well.  Every bfloat16 gradient element therefore lies within one rounding (2^-8
-    of its magnitude) of the float32 gradient on the widened inputs, plus what the float32 sums themselves vary
-    by: 1e-6 of the tensor's largest value for the order of the sums and of the float atomics, 1e-5 for
-    grad_input, whose terms pass through the fixed-point LDS cells (a grad column that differs in its last bit
-    may round to the neighbouring fixed-point step).  (The forward pass rounds its sampled columns to bfloat16
-    and is only close to the rounded float32 output.)"""
+def test_16bit_gradients_against_the_float32_gradients():
+    """backward_input_offset reads the 16-bit tensors itself and multiplies them in 16-bit matrix instructions
+    with float32 accumulation -- the products of 16-bit values are exact in float32, so only the order of the
+    sums differs from the float32 kernel -- and rounds each result once.  Every bfloat16 element of grad_input
+    and grad_offset therefore lies within one rounding (2^-8 of its magnitude) of the float32 gradient on the
+    widened inputs, plus what the float32 sums themselves vary by: 1e-6 of the tensor's largest value for the
+    order of the sums, 1e-5 for grad_input, whose terms pass through the fixed-point LDS cells (a grad column
+    that differs in its last bit may round to the neighbouring fixed-point step).  The forward pass and
+    backward_weight round their sampled columns to bfloat16 for the matrix instruction: output and grad_weight
+    are close to the float32 results (5e-3 of the largest value), not within one rounding."""
     import deform_conv3d_pytorch_op_amd as dcn
     c = make_case(*SMALL_CASES["3d_c4_like"], dtype=torch.bfloat16, seed=9)
     dev = torch.device("cuda:0")
@@ -88,11 +90,12 @@ def test_16bit_gradients_are_the_float32_gradients_rounded_once():
         out = dcn.ConvOffset3dFunction.apply(x, off, w, b, *cfg)
         out.backward(c["gout"].to(dev).to(dt))
         grads[dt] = (out.detach(), x.grad, off.grad, w.grad)
-    for name, g16, g32 in zip(("grad_input", "grad_offset", "grad_weight"), grads[torch.bfloat16][1:], grads[torch.float32][1:]):
+    for name, g16, g32 in zip(("grad_input", "grad_offset"), grads[torch.bfloat16][1:3], grads[torch.float32][1:3]):
         slack = 2.0 ** -8 * g32.abs() + (1e-5 if name == "grad_input" else 1e-6) * g32.abs().max()
         assert bool(((g16.float() - g32).abs() <= slack).all()), name
-    out16, out32 = grads[torch.bfloat16][0].float(), grads[torch.float32][0]
-    assert (out16 - out32).abs().max().item() <= 5e-3 * out32.abs().max().item()
+    for name, k in (("output", 0), ("grad_weight", 3)):
+        v16, v32 = grads[torch.bfloat16][k].float(), grads[torch.float32][k]
+        assert (v16 - v32).abs().max().item() <= 5e-3 * v32.abs().max().item(), name
 
 
 def test_oob_zero_switch_is_float_only():
