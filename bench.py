@@ -1,6 +1,6 @@
 """Benchmark of the deformable-convolution hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5|all] [--no-cpu] [--dtype f32|f64]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5|all] [--no-cpu] [--dtype f32|f64|bf16|f16]
 
 A step is one forward + backward (grad input, grad offset, grad weight) of one layer through the
 package's autograd Function on synthetic inputs already resident in HBM.  The default workload is
@@ -27,7 +27,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}     # MI355X dense matrix peaks
+PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6, "bfloat16": 2500.0, "float16": 2500.0}     # MI355X dense matrix peaks
+DTYPES = {"f32": "float32", "f64": "float64", "bf16": "bfloat16", "f16": "float16"}
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per C-ABI call measured with rocprofv3 (--pmc FETCH_SIZE, then --pmc WRITE_SIZE, each scaled by
@@ -102,7 +103,7 @@ def run_config(name, a):
 
     spec = CONFIGS[name]
     if a.dtype is not None:             # the configuration's shapes in the other precision
-        spec = spec[:-1] + ({"f32": "float32", "f64": "float64"}[a.dtype],)
+        spec = spec[:-1] + (DTYPES[a.dtype],)
     dtype = getattr(torch, spec[-1])
     kw = dict(dtype=dtype, seed=0, bias=False)
     if a.offset_scale is not None:      # not the configuration's own offsets: U[-s, s]
@@ -162,7 +163,7 @@ def run_config(name, a):
 
     # ---- per-kernel durations: each C-ABI call between two HIP events on its own stream ------
     L = _lib.load()
-    suf = "f32" if dtype == torch.float32 else "f64"
+    suf = {v: k for k, v in DTYPES.items()}[spec[-1]]
     geom = _geom(nd, x, w, c["outs"], c["stride"], c["pad"], c["dil"], c["cpg"], c["groups"])
     nbytes = L.dcn_workspace_bytes_for(x.element_size(), x.shape[0], x.shape[1], w.shape[0], math.prod(c["ins"]),
                                        math.prod(c["outs"]), math.prod(c["k"]), c["groups"], c["cpg"])
@@ -216,7 +217,7 @@ def run_config(name, a):
 
     # ---- CPU baseline: the oracle on a bounded sample of the same workload --------------------
     cpu = None
-    if not a.no_cpu:
+    if not a.no_cpu and a.dtype not in ("bf16", "f16"):      # (the oracle computes in float32 / float64)
         from oracle import dcn_oracle as orc
         ns = x.shape[0]
         xs, offs, gs = c["x"][:ns].contiguous(), c["off"][:ns].contiguous(), c["gout"][:ns].contiguous()
@@ -251,9 +252,10 @@ def run_config(name, a):
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_step, 4), "fwd_ms": round(ms_fwd, 4),
         "ms_per_step_events": step_events, "fwd_ms_events": fwd_events, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32" if dtype == torch.float32 else "f64", "data": "synthetic",
+        "vs_baseline": None, "dtype": suf, "data": "synthetic",
         "config": {"workload": name + ": " + DESCR[name] +
-                               ("" if a.dtype is None else " -- computed in %s instead of its own precision" % a.dtype) +
+                               ("" if a.dtype is None else " -- %s instead of its own precision" %
+                                ("stored as %s, float32 accumulation," % a.dtype if a.dtype in ("bf16", "f16") else "computed in %s" % a.dtype)) +
                                ("" if a.offset_scale is None else " -- with offsets U[-%g,%g] instead of its own" % (a.offset_scale, a.offset_scale))},
         "mfma_frac_whole_step": round(value / peak, 4),
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
@@ -269,8 +271,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--offset-scale", type=float, default=None,
                     help="offsets uniform in [-s, s] instead of the configuration's own (how the rates depend on the reach of the offsets)")
-    ap.add_argument("--dtype", choices=["f32", "f64"], default=None,
-                    help="run the configuration's shapes in this precision instead of its own (f64: against the fp64 matrix peak)")
+    ap.add_argument("--dtype", choices=sorted(DTYPES), default=None,
+                    help="run the configuration's shapes in this precision instead of its own (f64: against the fp64 matrix "
+                         "peak; bf16 / f16: tensors stored in 16 bits, float32 accumulation, against the 16-bit matrix peak)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic for scaling rocprof's "
                          "FETCH_SIZE / WRITE_SIZE counters)")

@@ -1332,15 +1332,29 @@ int backward_weight_native16(const Params& Pin, const S* in, const S* off, const
     if ((unsigned long long)P.inV * P.C_in * sizeof(S) >= (1ull << 32) || (unsigned long long)P.outV * P.C_out >= (1ull << 32)) return DCN_OK;
     if (2 * (long long)P.N > 65535) return DCN_OK;
     const int mtiles = (P.M + TN - 1) / TN;
-    const int MT = mtiles >= 2 ? 2 : 1;             // (four row tiles would take 128 accumulator registers beside the two channel tiles)
+    // Two row tiles per workgroup at most (four would take 128 accumulator registers beside the two
+    // channel tiles: one wavefront per SIMD), so more than 64 output channels sample everything once
+    // per 64 of them, and channel segments that fill their 64-channel tiles badly waste the lanes'
+    // loads.  Both kernels are bounded by their corner loads: this one issues half as many per
+    // channel as the float32 kernel (four row tiles, 32-channel tiles), times the re-sampling and the
+    // unused part of the tiles.  Where that comes to more than the float32 kernel's, that kernel on
+    // widened tensors is the faster one (128 -> 128 channels in deformable groups of 32, 3-D: 2.5 ms
+    // here against 1.2 + 0.15 for widening; 256 -> 256 in one group, 2-D: 0.20 here against 0.31).
+    const int MT = mtiles >= 2 ? 2 : 1;
     P.mchunks = (mtiles + MT - 1) / MT;
     P.nctiles = 0;
+    int nct32 = 0;
     for (int gg = 0; gg < P.G; ++gg) {
         const int cg0 = gg * P.Cg, cg1 = cg0 + P.Cg;
         for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
             const int cb = cg0 > dg * P.cpg ? cg0 : dg * P.cpg, ce = cg1 < (dg + 1) * P.cpg ? cg1 : (dg + 1) * P.cpg;
             P.nctiles += (ce - cb + CT - 1) / CT;
+            nct32 += (ce - cb + TN - 1) / TN;
         }
+    }
+    {
+        const long long loads16 = (long long)P.mchunks * P.nctiles, loads32 = (long long)((mtiles + 3) / 4) * nct32;
+        if (4 * loads16 > 5 * loads32) return DCN_OK;
     }
     // position splits: about 2560 workgroups, as in the float kernel's plan
     const long long slabs = (long long)P.N * ((P.outV + TN - 1) / TN), other = (long long)P.kV * P.nctiles * P.mchunks;
