@@ -284,6 +284,10 @@ static int forward_tail_split() {       // DCN_FORWARD_TAIL=0: the forward pass 
     static const int v = [] { const char* e = getenv("DCN_FORWARD_TAIL"); return e ? atoi(e) : 1; }();
     return v;
 }
+static bool forward_tail_two_runs() {    // DCN_FORWARD_TAIL2=0: the split units of the forward pass's last round are all split the same number of ways
+    static const int v = [] { const char* e = getenv("DCN_FORWARD_TAIL2"); return (e && atoi(e) == 0) ? 0 : 1; }();
+    return v != 0;
+}
 static bool fused_pair() {              // DCN_FUSED_PAIR=0: float32 LDS cells of the fused backward kernel hold one channel each (64-bit)
     static const int v = [] { const char* e = getenv("DCN_FUSED_PAIR"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
@@ -604,62 +608,103 @@ int forward(const Geometry& g, const S* in, const S* w, const S* off, const S* b
                 if (l > lds) lds = l;
             }
             const Params& Ph = plans[0];
-            using Kern = void (*)(Params, PlanSet, const unsigned*, const S*, const S*, const S*, const S*, S*, T*, int, unsigned);
+            using Kern = void (*)(Params, PlanSet, const unsigned*, const S*, const S*, const S*, const S*, S*, T*, int, unsigned, TailSplit);
             Kern kern;
             if (nw == 16) kern = MT == 1 ? forward_quad_kernel<T, ND, 1, 16, S> : forward_quad_kernel<T, ND, 2, 16, S>;
             else kern = MT == 1 ? forward_quad_kernel<T, ND, 1, WAVESH, S> : MT == 2 ? forward_quad_kernel<T, ND, 2, WAVESH, S>
                       : MT == 4 ? forward_quad_kernel<T, ND, 4, WAVESH, S> : forward_quad_kernel<T, ND, 8, WAVESH, S>;
             T* part = reinterpret_cast<T*>(static_cast<char*>(ws) + align256(wq_bytes));      // partial sums, in the arithmetic type
             // A grid that ends in a partly filled round of workgroups: the units of that round, last in
-            // the launch, are split over tsplit workgroups each (every tsplit-th channel pass), so that
-            // the round fills the device; forward_join_tail_kernel adds their partial sums.  A
-            // workgroup's fixed part (halo table, offsets, output) is charged as 5 % of a unit.
+            // the launch, are split over several workgroups each (every tsplit-th channel pass), so that
+            // the round fills the device; forward_join_tail_kernel adds their partial sums.  Either all
+            // of them tsplit ways, or -- when that leaves the last of the resulting short rounds partly
+            // empty -- as many of them tsplit + 1 ways as make the workgroup count a whole number of
+            // rounds (TailSplit: the units split tsplit ways come first, so that the longer workgroups
+            // start first).  Cost of a workgroup: per channel pass one part for the tap geometry and one
+            // per four channels, plus 5 % of a unit for its fixed part (halo table, offsets, output).
             const long long units = (long long)Ph.N * Ph.tiles * Ph.G * Ph.mchunks;
             int tsplit = 1;
             long long whole = 0;
+            TailSplit ts = {0u, 0, 0};
             if (fsplit == 1 && forward_tail_split()) {
                 const long long slots = forward_slots() ? forward_slots() : resident_workgroups(reinterpret_cast<const void*>(kern), nw * 64, lds);
                 const long long rest = units % slots;
+                constexpr double GEO = 0.45;    // tap geometry of a pass, in units of four channels' sampling and contraction
+                // cost of the longest workgroup when the passes of a unit (cch channels each) are dealt to cs workgroups
+                auto wg_cost = [&](int cs, int cch, int* npasses) {
+                    double load[64] = {0};
+                    int k = 0;
+                    for (int dg = 0; dg <= (P.Cg - 1) / P.cpg; ++dg) {
+                        const int len = (P.Cg < (dg + 1) * P.cpg ? P.Cg : (dg + 1) * P.cpg) - dg * P.cpg;
+                        for (int c0 = 0; c0 < len; c0 += cch, ++k) load[k % cs] += GEO + (double)(((len - c0 < cch ? len - c0 : cch) + FQ - 1) / FQ);
+                    }
+                    if (npasses) *npasses = k;
+                    double worst = 0;
+                    for (int z = 0; z < cs; ++z) worst = load[z] > worst ? load[z] : worst;
+                    return worst;
+                };
                 int passes = 0;                 // channel passes of a unit under the first plan
-                for (int dg = 0; dg <= (P.Cg - 1) / P.cpg; ++dg) {
-                    const int len = (P.Cg < (dg + 1) * P.cpg ? P.Cg : (dg + 1) * P.cpg) - dg * P.cpg;
-                    passes += (len + Ph.cchunk - 1) / Ph.cchunk;
-                }
+                const double unit_cost = wg_cost(1, Ph.cchunk, &passes);
                 const size_t end = pc.sel ? (ws_bytes - 256) / 256 * 256 : ws_bytes;
                 const size_t room = end > align256(wq_bytes) ? end - align256(wq_bytes) : 0;
+                const size_t per_wg = (size_t)MT * TN * nw * TN * sizeof(T);
                 if (units > slots && rest) {
                     double best = 0.9;          // of the time of an unsplit last round; a tenth must be gained
                     for (int cs = 2; cs <= 8 && cs <= passes; ++cs) {
-                        const double t = (double)((rest * cs + slots - 1) / slots) * ((double)((passes + cs - 1) / cs) / passes + 0.05);
-                        const size_t bytes = (size_t)rest * cs * MT * TN * nw * TN * sizeof(T);
                         if (forward_tail_split() > 1 && cs != forward_tail_split()) continue;
-                        if ((t < best || forward_tail_split() > 1) && bytes <= room && bytes <= FWD_PARTIAL_CAP) { best = t; tsplit = cs; }
+                        const long long rounds = (rest * cs + slots - 1) / slots;
+                        const double ta = wg_cost(cs, Ph.cchunk, nullptr) / unit_cost + 0.05;
+                        {
+                            const double t = (double)rounds * ta;
+                            const size_t bytes = (size_t)rest * cs * per_wg;
+                            if ((t < best || forward_tail_split() > 1) && bytes <= room && bytes <= FWD_PARTIAL_CAP) {
+                                best = t; tsplit = cs; ts = TailSplit{0u, 0, 0};
+                            }
+                        }
+                        // two runs: nb units cs + 1 ways, the others cs ways, rounds * slots workgroups in all;
+                        // the cs-way workgroups must fit the first round
+                        const long long nb = rounds * slots - rest * cs;
+                        if (!forward_tail_two_runs() || cs + 1 > 8 || nb <= 0 || nb >= rest || (rest - nb) * cs > slots) continue;
+                        double tb = 1e30;
+                        int cchb = Ph.cchunk;
+                        for (int cch = Ph.cchunk; cch >= FQ; cch -= FQ) {
+                            int np = 0;
+                            const double c = wg_cost(cs + 1, cch, &np) / unit_cost + 0.05;
+                            if (np >= cs + 1 && c < tb) { tb = c; cchb = cch; }
+                        }
+                        const double t = ta + (double)(rounds - 1) * tb;
+                        const size_t bytes = (size_t)(rounds * slots) * per_wg;
+                        if (t < best && bytes <= room && bytes <= FWD_PARTIAL_CAP) {
+                            best = t; tsplit = cs; ts = TailSplit{(unsigned)(rest - nb), cs + 1, cchb};
+                        }
                     }
                     if (tsplit > 1) whole = units - rest;
                 }
             }
-            const long long wgs = tsplit > 1 ? whole + (units - whole) * tsplit : units * fsplit;
+            const long long wgs = tsplit > 1 ? whole + (ts.splitB ? (long long)ts.unitsA * tsplit + (units - whole - ts.unitsA) * ts.splitB : (units - whole) * tsplit)
+                                             : units * fsplit;
             if (wgs > 0x7fffffffLL) return fail(DCN_E_ARGUMENT, "too many workgroups for one launch");
             const dim3 grid((unsigned)wgs);
             if (trace_plans()) {
                 fprintf(stderr, "dcn forward: %d wavefronts, MT %d, grid %u (%lld unsplit, rest x %d), LDS %zu, every unit split x %d\n", nw, MT, grid.x,
                         tsplit > 1 ? whole : 0LL, tsplit, lds, fsplit);
+                if (ts.splitB) fprintf(stderr, "  of the rest: %u units x %d, the others x %d with %d channels per pass\n", ts.unitsA, tsplit, ts.splitB, ts.cchB);
                 for (int k = 0; k < pc.nplans; ++k)
                     fprintf(stderr, "  plan %d: margin %d, halo %d x %d x %d, %d channels per pass, base cost %.3f\n", k, pc.margin[k],
                             plans[k].hext[0], plans[k].hext[1], plans[k].hext[2], plans[k].cchunk, pc.base[k]);
             }
             const unsigned* sel = pc.sel;
             if (int rc = launch_halo(kern, "forward_quad_kernel", grid, nw * 64, lds, s, Ph, alts, sel, in, off, (const S*)wt, bias, out, part,
-                                     tsplit > 1 ? tsplit : fsplit, (unsigned)whole))
+                                     tsplit > 1 ? tsplit : fsplit, (unsigned)whole, ts))
                 return rc;
             if (fsplit == 1 && tsplit == 1) return DCN_OK;
             if (tsplit > 1) {
-                using Join = void (*)(Params, PlanSet, const unsigned*, const T*, const S*, S*, int, unsigned);
+                using Join = void (*)(Params, PlanSet, const unsigned*, const T*, const S*, S*, int, unsigned, TailSplit);
                 Join join;
                 if (nw == 16) join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, 16, S> : forward_join_tail_kernel<T, ND, 2, 16, S>;
                 else join = MT == 1 ? forward_join_tail_kernel<T, ND, 1, WAVESH, S> : MT == 2 ? forward_join_tail_kernel<T, ND, 2, WAVESH, S>
                           : MT == 4 ? forward_join_tail_kernel<T, ND, 4, WAVESH, S> : forward_join_tail_kernel<T, ND, 8, WAVESH, S>;
-                hipLaunchKernelGGL(join, dim3((unsigned)((units - whole) * (MT * TN / JOIN_ROWS))), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole);
+                hipLaunchKernelGGL(join, dim3((unsigned)((units - whole) * (MT * TN / JOIN_ROWS))), dim3(nw * TN), 0, s, Ph, alts, sel, (const T*)part, bias, out, tsplit, (unsigned)whole, ts);
                 return check_launch("forward_join_tail_kernel");
             }
             if constexpr (!S16) {

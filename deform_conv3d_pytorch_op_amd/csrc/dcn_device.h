@@ -50,6 +50,14 @@ struct PlanSet {
     HaloPlan alt[MAX_PLANS - 1];  // plans 1 .. MAX_PLANS - 1 (plan 0 is the Params argument itself)
     unsigned mask;                // bit i: this launch runs plan i
 };
+// The split units at the end of a forward launch (after `whole` unsplit ones) come in two runs: the
+// first unitsA units are split `csplit` ways (the kernel argument), the others splitB ways, with at
+// most cchB channels per LDS pass so that their workgroups get equal shares (splitB = 0: one run).
+// Their workgroups follow in that order, and so do their partial sums.
+struct TailSplit {
+    unsigned unitsA;
+    int splitB, cchB;
+};
 struct PlanChoice {
     unsigned* sel;                // chosen plan (device memory), null: a single plan, nothing to choose
     int nplans, nd;

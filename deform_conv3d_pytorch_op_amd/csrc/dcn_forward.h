@@ -101,7 +101,8 @@ __device__ inline void halo_stage_quads(const Params& P, const HaloPlan& H, cons
 //   whole > 0 (a grid that ends in a partly filled round of workgroups): the first `whole` units
 //     run unsplit and write the output itself, the others, last in the launch, are split so that
 //     the last round fills the device; their partial sums go to part as
-//     [unit - whole][cz][row of the chunk][position of the block] (forward_join_tail_kernel).
+//     [split workgroup][row of the chunk][position of the block] in launch order, i.e.
+//     [unit - whole][cz] within each of the two runs of TailSplit (forward_join_tail_kernel).
 // (few accumulators: four wavefronts per SIMD, i.e. at most 128 registers, also for the 512-thread
 // shape, so that two of its workgroups share a CU)
 // S: storage format of the tensors (see Store); T is float with a 16-bit format, and partial sums are always T.
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
                                                            const S* __restrict__ in,
                                                            const S* __restrict__ off, const S* __restrict__ Wq,
                                                            const S* __restrict__ bias, S* __restrict__ out,
-                                                           T* __restrict__ part, int csplit, unsigned whole) {
+                                                           T* __restrict__ part, int csplit, unsigned whole, TailSplit ts) {
     HaloPlan H;
     if (!chosen_halo(P, alts, sel, H)) return;          // another launch runs the chosen plan
     using MM = Mma<T>;
@@ -124,14 +125,27 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % TN, q = lane / TN;
     // workgroups of one tile are neighbours in an XCD-contiguous order
-    unsigned wg;
+    unsigned wg, pslot = 0;                             // pslot: which partial sum of the split runs
     int cz = 0;
+    int cch = H.cchunk;                                 // channels per LDS pass
     const bool split = csplit > 1 && blockIdx.x >= whole;
     if (!split) wg = xcd_contiguous(blockIdx.x, csplit > 1 ? whole : gridDim.x);
     else {
-        const unsigned r = xcd_contiguous(blockIdx.x - whole, gridDim.x - whole);
-        wg = whole + r / (unsigned)csplit;
-        cz = r % (unsigned)csplit;
+        const unsigned rel = blockIdx.x - whole, all = gridDim.x - whole;
+        const unsigned wgsA = ts.splitB ? ts.unitsA * (unsigned)csplit : all;
+        if (rel < wgsA) {
+            const unsigned r = xcd_contiguous(rel, wgsA);
+            wg = whole + r / (unsigned)csplit;
+            cz = r % (unsigned)csplit;
+            pslot = r;
+        } else {
+            const unsigned r = xcd_contiguous(rel - wgsA, all - wgsA);
+            csplit = ts.splitB;
+            wg = whole + ts.unitsA + r / (unsigned)csplit;
+            cz = r % (unsigned)csplit;
+            pslot = wgsA + r;
+            cch = min(cch, ts.cchB);
+        }
     }
     if (!split) csplit = 1;
     const unsigned gm = wg % (unsigned)(P.G * P.mchunks);
@@ -173,9 +187,9 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     for (int dg = cg0 / P.cpg; dg <= (cg1 - 1) / P.cpg; ++dg) {
         const int cb = max(cg0, dg * P.cpg), ce = min(cg1, (dg + 1) * P.cpg);
         const S* off_dg = off + ((size_t)n * P.DG + dg) * P.kV * ND * P.outV;
-        for (int cc0 = cb; cc0 < ce; cc0 += H.cchunk) {
+        for (int cc0 = cb; cc0 < ce; cc0 += cch) {
             if ((chunk_no++) % csplit != cz) continue;                     // another workgroup's chunk (uniform)
-            const int nch = min(H.cchunk, ce - cc0);
+            const int nch = min(cch, ce - cc0);
             const int ngrp = (nch + FQ - 1) / FQ;
             const S* chan0 = in + ((size_t)n * P.C_in + cc0) * P.inV;      // workgroup-uniform
             if (threadIdx.x == 0) sNonFinite = 0;
@@ -362,8 +376,8 @@ __global__ __launch_bounds__(NW * 64, (MT <= 2 && sizeof(T) == 4) ? 4 : 1) void 
     }
 
     if (split && whole > 0) {
-        // partial sums of a unit of the last round: [unit - whole][cz][MT * TN rows][NW * TN positions]
-        T* dst = part + ((size_t)(wg - whole) * csplit + cz) * (MT * TN) * (NW * TN) + wave * TN + j;
+        // partial sums of a unit of the last round: [split workgroup][MT * TN rows][NW * TN positions]
+        T* dst = part + (size_t)pslot * (MT * TN) * (NW * TN) + wave * TN + j;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -397,7 +411,7 @@ constexpr int JOIN_ROWS = 8;
 template <typename T, int ND, int MT, int NW, typename S = T>
 __global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, PlanSet alts, const unsigned* __restrict__ sel,
                                                                     const T* __restrict__ part, const S* __restrict__ bias,
-                                                                    S* __restrict__ out, int csplit, unsigned whole) {
+                                                                    S* __restrict__ out, int csplit, unsigned whole, TailSplit ts) {
     constexpr int TN = Mma<T>::TN, SLICES = MT * TN / JOIN_ROWS;
     static_assert(MT * TN % JOIN_ROWS == 0, "row slices");
     HaloPlan H;
@@ -412,7 +426,12 @@ __global__ __launch_bounds__(NW * 64) void forward_join_tail_kernel(Params P, Pl
     int o[ND];
     unsigned pos;
     if (!tile_position<ND>(P, tg_, (int)threadIdx.x, o, pos)) return;
-    const T* src = part + ((size_t)unit * csplit * (MT * TN) + ml0) * (NW * TN) + threadIdx.x;
+    size_t first = (size_t)unit * csplit;               // the unit's first partial sum
+    if (ts.splitB && unit >= ts.unitsA) {
+        first = (size_t)ts.unitsA * csplit + (size_t)(unit - ts.unitsA) * ts.splitB;
+        csplit = ts.splitB;
+    }
+    const T* src = part + (first * (MT * TN) + ml0) * (NW * TN) + threadIdx.x;
     T v[JOIN_ROWS];
 #pragma unroll
     for (int r = 0; r < JOIN_ROWS; ++r) v[r] = src[(size_t)r * (NW * TN)];
