@@ -844,10 +844,12 @@ template <> struct LdsCell<float> {
     // rounded product in its low mantissa bits (|term| < 2^22, which the caller's scale ensures).
     static constexpr float MAGIC32 = 12582912.f;             // 1.5 * 2^23, bit pattern 0x4B400000
     __device__ static inline void add2(type* p, float w, float g0_scaled, float g1_scaled) {
-        const int a = (int)(__float_as_uint(__builtin_fmaf(w, g0_scaled, MAGIC32)) - 0x4B400000u);
-        const int b = (int)(__float_as_uint(__builtin_fmaf(w, g1_scaled, MAGIC32)) - 0x4B400000u) + (a >> 31);
-        const type v = ((type)(unsigned)b << 32) | (type)(unsigned)a;
-        (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        // one 64-bit subtraction strips the constant from both halves; its borrow out of the low half
+        // (exactly when a is negative) is the lowering of b by one
+        typedef float F2 __attribute__((ext_vector_type(2)));
+        const F2 t = {__builtin_fmaf(w, g0_scaled, MAGIC32), __builtin_fmaf(w, g1_scaled, MAGIC32)};
+        const type raw = __builtin_bit_cast(type, t);
+        (void)__hip_atomic_fetch_add(p, raw - 0x4B4000004B400000ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     __device__ static inline void value2(type c, double inv_scale, float& v0, float& v1) {
         const int a = (int)(unsigned)c;
