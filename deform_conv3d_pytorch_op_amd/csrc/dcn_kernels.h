@@ -1561,7 +1561,7 @@ __global__ __launch_bounds__(NW * 64) void backward_input_halo_kernel(Params P, 
                             const T* ip = sIn + (size_t)base * CCH;
                             constexpr int GPV = swizzle_groups<T, CCH>();
                             if constexpr (GPV > 1) {
-                                // the four-channel group of this round sits at slot (group ^ voxel mod GPV) of its
+                                // the four-channel group read here sits at slot (group ^ voxel mod GPV) of its
                                 // voxel (halo_stage_interleaved); the innermost halo extent is a multiple of GPV
                                 // (host), so a corner's voxel is base + (i & 1) modulo GPV
                                 static_assert(RW == 4, "a round reads one four-channel group");
