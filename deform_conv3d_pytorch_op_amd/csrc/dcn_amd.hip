@@ -186,6 +186,7 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_FORWARD_WG=512     never use the 1024-thread forward variant; =1024 use it whenever its halo fits
 //   DCN_FORWARD_SPLIT=n    forward pass: split the input channels of a position block over at most n workgroups (0: never)
 //   DCN_FORWARD_TAIL=0     forward pass: never split only the units of the last, partly filled round of workgroups (n > 1: n ways)
+//   DCN_FORWARD_TAIL2=0    forward pass: the split units of the last round all the same number of ways, never in two runs
 //   DCN_FORWARD_SLOTS=n    forward pass: plan the launch as if n workgroups ran at once (test hook)
 //   DCN_SCATTER_BUDGET_KB  LDS per workgroup of the privatised scatter kernel (default 144)
 //   DCN_SCATTER=global     scatter grad-input with global atomics instead of the LDS-privatised kernel
@@ -197,6 +198,9 @@ int relayout(const Params& P, const T* w, T* wt, int channel_fastest, hipStream_
 //   DCN_FUSED_SLOTS=n      fused backward kernel: plan the launch as if n workgroups ran at once (test hook)
 //   DCN_FUSED_FIXED=0      fused backward kernel: runtime plane stride even where the compile-time one fits
 //   DCN_FUSED_PAIR=0       fused backward kernel, float32: one channel per 64-bit LDS cell instead of two 32-bit halves
+//   DCN_FUSED_BREG2=0      fused backward kernel: no second register set for the grad_output operand of 64 < M <= 128
+//   DCN_GLOBAL_PLAN=0      backward_input_offset (3-D): the device is not offered the path without LDS tiling
+//   DCN_NATIVE16=0         16-bit entry points: always widen to float32 and run the float32 kernels
 static size_t env_kb(const char* name, int dflt) {
     const char* e = getenv(name);
     const int v = e ? atoi(e) : dflt;
@@ -296,7 +300,7 @@ static bool fused_breg2() {             // DCN_FUSED_BREG2=0: grad_output operan
     static const int v = [] { const char* e = getenv("DCN_FUSED_BREG2"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
 }
-static bool native16() {                // DCN_NATIVE16=0: the 16-bit forward entry points always widen to float32 first
+static bool native16() {                // DCN_NATIVE16=0: the 16-bit entry points always widen to float32 first
     static const int v = [] { const char* e = getenv("DCN_NATIVE16"); return (e && atoi(e) == 0) ? 0 : 1; }();
     return v != 0;
 }
