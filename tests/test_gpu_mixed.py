@@ -66,9 +66,11 @@ def test_16bit_storage_medium_cases_match_oracle(name, dtype):
     _compare(make_case(*MEDIUM[name], dtype=dtype, seed=8), dtype, name)
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(160))
 def test_16bit_storage_random_geometries_match_oracle(seed):
-    """Seeded random small (even seeds) and medium (odd seeds) geometries in both 16-bit formats."""
+    """Seeded random small (even seeds) and medium (odd seeds) geometries in both 16-bit formats.
+    (Seeds 33, 91, 93, 119, 141, 149 hold 16-bit offsets of about -1e-6 beside integer coordinates: single
+    samples there differ from an oracle with float64 coordinates, see the module text.)"""
     spec = random_spec(seed, medium=bool(seed % 2))
     print("16-bit random geometry", seed, spec, flush=True)
     for dtype in (torch.bfloat16, torch.float16):

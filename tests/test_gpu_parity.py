@@ -70,7 +70,7 @@ def test_small_cases_match_oracle(name, dtype):
     compare(c, dtype, name)
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(96))
 def test_random_geometries_match_oracle(seed):
     """Seeded random small geometries (2-D / 3-D, odd channel counts, all divisors as deformable-group
     widths, rectangular kernels, per-axis stride / padding / dilation), float64 and float32."""
@@ -80,7 +80,7 @@ def test_random_geometries_match_oracle(seed):
         compare(make_case(*spec, dtype=dtype, seed=100 + seed), dtype, "random_%d" % seed)
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(48))
 def test_random_medium_geometries_match_oracle(seed):
     """The same with extents of several position tiles per axis (halo tiling, channel splits, partial
     tiles at the rim) and up to 72 input channels."""
