@@ -209,8 +209,14 @@ int conv2d_backward_weight_f64(const double *input, const double *grad_output, d
  * format and multiplied with the weights by 16-bit matrix instructions that accumulate in float32;
  * bias added in float32, one rounding per output element.  (Layers that the LDS-halo kernel cannot
  * serve are widened to float32 and computed there.)
- * backward_*: the values are widened exactly, all products and sums are the float32 kernels', and
- * each result element is rounded once, to nearest even.
+ * backward_input_offset: the fused kernel reads the 16-bit tensors itself and forms the grad columns
+ * with 16-bit matrix instructions (products of 16-bit values are exact in float32; float32 sums);
+ * coordinates, interpolation, the scatter and the coordinate gradient are float32.
+ * backward_weight: like forward, the sampled columns are rounded to the storage format and multiplied
+ * with grad_output by 16-bit matrix instructions that accumulate in float32.
+ * Each result element is rounded once, to nearest even.  Layers that these kernels do not serve (more
+ * output channels than the fused kernel keeps in registers, odd channel counts, ...) are widened exactly
+ * into float32 copies and computed by the float32 kernels, with the same single rounding at the end.
  * Same argument meaning and accumulate / overwrite contract as the _f32 calls (grad_input and
  * grad_weight: rounded sum of their previous content and the gradient).  The workspace must come
  * from dcn_workspace_bytes_for(2, ...): it also holds float copies of the tensors.  Offsets in 16
