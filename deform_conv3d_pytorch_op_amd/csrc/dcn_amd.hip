@@ -1276,9 +1276,11 @@ int backward_weight(const Geometry& g, const T* in, const T* off, const T* gout,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Mixed precision: tensors stored as bfloat16 / binary16, arithmetic in float32.  The tensors are
-// widened into float copies at the front of the workspace, the float32 kernels run on them with the
-// rest of the workspace, and the results are rounded once.
+// Mixed precision: tensors stored as bfloat16 / binary16, accumulation in float32.  Each call first
+// offers the layer to the kernel that reads the 16-bit tensors itself and multiplies on the 16-bit
+// matrix instructions (float results in a float copy at the front of the workspace, rounded once
+// when they are written back); where that kernel declines, the tensors are widened into float
+// copies at the front of the workspace and the float32 kernels run on them with the rest of it.
 struct Carver {
     char* p;
     size_t left;
